@@ -1,0 +1,202 @@
+/*
+ * sddmm.h -- C ABI of the MI355X (gfx950) SDDMM engine.
+ *
+ *   out[p] = S.val[p] * dot(W[row_p, 0:K], H[col_p, 0:K])     for every nonzero p of S
+ *
+ * S is a (row, col)-sorted sparse matrix with int32 indices and fp32 values,
+ * W is n_rows x K and H is n_cols x K, both fp32 row-major; out has one fp32
+ * per nonzero, in the order of the sorted S.
+ *
+ * The reference program (isratnisa/SDDMM_GPU) has no library interface: it is
+ * one translation unit whose main() calls free functions.  Each entry point
+ * below replaces one of those call sites; the citation names the reference
+ * lines (relative to HiPC18/src/).  All functions return SDDMM_OK (0) or an
+ * error code and never throw; sddmm_last_error() gives the message of the
+ * last failure on the calling thread.  "host" / "device" say where a pointer
+ * must live.  Plans are immutable after creation: sddmm_execute may be called
+ * from several threads on the same plan (each call on its own stream).
+ */
+#ifndef SDDMM_H
+#define SDDMM_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    SDDMM_OK = 0,
+    SDDMM_ERR_ARG = 1,      /* null pointer, non-positive size, K < 1, ... */
+    SDDMM_ERR_IO = 2,       /* file cannot be opened / read / written */
+    SDDMM_ERR_FORMAT = 3,   /* not a coordinate Matrix Market file, short file, bad token */
+    SDDMM_ERR_RANGE = 4,    /* an index outside the matrix, or sizes beyond int32 offsets */
+    SDDMM_ERR_UNSORTED = 5, /* operation needs a (row, col)-sorted matrix */
+    SDDMM_ERR_HIP = 6,      /* a HIP runtime call failed, or no gfx950 device */
+    SDDMM_ERR_NOMEM = 7
+};
+
+/* Kernel families a plan can be pinned to (sddmm_plan_create flags, low byte).
+ * AUTO lets the planner choose from the matrix shape, K and the tile sizes. */
+enum {
+    SDDMM_KERNEL_AUTO = 0,
+    SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM */
+    SDDMM_KERNEL_LDS_TILE = 2    /* column tiles of H staged in LDS, W row in VGPRs */
+};
+
+typedef struct sddmm_coo sddmm_coo;   /* host-side sparse matrix (COO, int32/int32/fp32) */
+typedef struct sddmm_plan sddmm_plan; /* device-side execution plan for one (S pattern, K, tiles) */
+
+typedef struct sddmm_plan_info {
+    int64_t n_rows, n_cols, nnz;
+    int64_t rows_touched, cols_touched; /* rows / columns with at least one nonzero */
+    int32_t K;
+    int32_t tile_size_x;  /* columns of S (= rows of H) per LDS tile actually used */
+    int32_t tile_size_y;  /* row-panel height actually used */
+    int32_t k_slice;      /* K elements of each H row resident in LDS at a time (== K: no slicing) */
+    int32_t n_col_tiles, n_row_panels;
+    int32_t kernel;       /* SDDMM_KERNEL_* actually chosen */
+    int32_t lanes_per_nnz;
+    int32_t lds_bytes;    /* LDS per workgroup of the main kernel */
+    int32_t grid, block;  /* launch shape of the main kernel */
+    int64_t n_blocks;     /* (row panel, column tile) work items with at least one nonzero */
+    int64_t device_bytes; /* device memory owned by the plan */
+    double plan_ms;       /* host time spent in the tiling pass + upload */
+} sddmm_plan_info;
+
+const char *sddmm_last_error(void);
+const char *sddmm_version(void);
+
+/* ---------------------------------------------------------------- input --- */
+
+/* Reads a Matrix Market coordinate file (real | integer | pattern, general |
+ * symmetric; '%' comment lines; the banner line may be missing).  Indices
+ * become 0-based.  Order and duplicates are kept as in the file.
+ * Replaces the inline reader in main(), sddmm.cu:257-283.                   */
+int sddmm_read_mtx(const char *path, sddmm_coo **out);
+
+/* Writes S as "%%MatrixMarket matrix coordinate real general" (1-based). */
+int sddmm_write_mtx(const sddmm_coo *S, const char *path);
+
+/* Binary side-file of a parsed matrix (header + raw arrays), so large inputs
+ * are parsed from text once.  The reference's analogue is the ad-hoc text
+ * dump at util.h:83-118.                                                    */
+int sddmm_write_bin(const sddmm_coo *S, const char *path);
+int sddmm_read_bin(const char *path, sddmm_coo **out);
+
+/* Copies caller arrays (host) into a new matrix.  vals may be NULL (all 1). */
+int sddmm_coo_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *rows,
+                     const int32_t *cols, const float *vals, sddmm_coo **out);
+void sddmm_coo_destroy(sddmm_coo *S);
+
+int sddmm_coo_info(const sddmm_coo *S, int64_t *n_rows, int64_t *n_cols, int64_t *nnz,
+                   int *is_row_col_sorted);
+/* Borrowed host pointers, valid until S is modified or destroyed. */
+int sddmm_coo_arrays(const sddmm_coo *S, const int32_t **rows, const int32_t **cols,
+                     const float **vals);
+
+/* Stable sort into (row, col) order; duplicates kept in file order. */
+int sddmm_coo_sort_rows(sddmm_coo *S);
+
+/* "Conversion from col sorted to row sorted": swaps the roles of rows and
+ * columns (n_rows <-> n_cols) and sorts, so a column-sorted file of A comes
+ * out as row-sorted A^T.  Replaces unsorted_make_CSR, util.h:82-128.        */
+int sddmm_coo_transpose_sort(sddmm_coo *S);
+
+/* CSR row pointers (n_rows+1 entries, host) of a sorted matrix. */
+int sddmm_coo_row_ptr(const sddmm_coo *S, int32_t *row_ptr);
+
+/* Compressed CSR over the non-empty rows: row_holder[h] = h-th non-empty row,
+ * row_ptr[h]..row_ptr[h+1] its nonzeros.  row_ptr has room for n_rows+1,
+ * row_holder for n_rows entries.  Replaces make_CSR, util.h:131-153.        */
+int sddmm_coo_compress_rows(const sddmm_coo *S, int32_t *row_ptr, int32_t *row_holder,
+                            int64_t *n_nonempty);
+
+/* X[r*k+t] = 0.1*drand48() after srand48(0): the dense factors the reference
+ * CLI runs with.  Replaces initial(), util.h:75-81.  X is a host pointer.   */
+int sddmm_init_reference(float *X, int64_t n, int32_t k);
+
+/* --------------------------------------------------------------- tiling --- */
+
+/* Host-side result of the tiling pass, for inspection and tests.  S is cut
+ * into column tiles of tile_size_x columns; "tile order" lists the nonzeros
+ * tile by tile, rows ascending inside a tile, columns ascending inside a row
+ * -- the order rewrite_matrix_1D writes (util.h:267-343).  Nonzeros are not
+ * copied: tiled_ind gives, for each tile-order position, the position in the
+ * sorted S (the reference's tiled_ind, util.h:301).  Because S is (row, col)-
+ * sorted, each (tile, row) run is a contiguous range of original positions.
+ * Inside a tile every tile_size_y active rows (rows with a nonzero in the
+ * tile) form a row panel; block_end holds the tile-order end offset of each
+ * panel (the reference's lastIdx_block_tile, stored without its n_rows/Y+1
+ * stride).  Replaces TiledMatrix + rewrite_matrix_1D, util.h:33-66, 267-343. */
+typedef struct sddmm_tiling sddmm_tiling;
+typedef struct sddmm_tiling_view {
+    int32_t tile_size_x, tile_size_y, n_col_tiles;
+    int32_t max_active_rows;   /* largest n_actv_row: rewrite_matrix_1D's return value */
+    int64_t nnz;
+    const int32_t *tile_ptr;   /* [n_col_tiles+1] tile-order offsets (lastIdx_tile) */
+    const int32_t *tiled_ind;  /* [nnz] */
+    const int64_t *active_ptr; /* [n_col_tiles+1]; n_actv_row[j] = active_ptr[j+1]-active_ptr[j] */
+    const int32_t *active_row; /* global row ids, tile j at [active_ptr[j], active_ptr[j+1]) */
+    const int32_t *active_end; /* tile-order end offset of that row's run */
+    const int64_t *block_ptr;  /* [n_col_tiles+1] offsets into block_end */
+    const int32_t *block_end;  /* tile-order end offset of each row panel */
+} sddmm_tiling_view;
+int sddmm_tiling_create(const sddmm_coo *S, int32_t tile_size_x, int32_t tile_size_y,
+                        sddmm_tiling **out);
+int sddmm_tiling_get(const sddmm_tiling *T, sddmm_tiling_view *view);
+void sddmm_tiling_destroy(sddmm_tiling *T);
+
+/* ----------------------------------------------------------------- plan --- */
+
+/* Builds a plan from a sorted host matrix: runs the tiling pass for
+ * (K, tile_size_x, tile_size_y), uploads index arrays and S.val.  tile sizes
+ * of 0 mean "choose".  tile_size_x = columns of S per LDS tile, tile_size_y =
+ * row-panel height: the 3rd and 4th positional arguments of the reference CLI
+ * (README.md:21-33).  flags: low byte = SDDMM_KERNEL_*.
+ * Replaces the TiledMatrix/rewrite_matrix_1D call in preprocessing()
+ * (sddmm.cu:208-232) and the allocation + host-to-device part of sddmm_GPU
+ * (sddmm.cu:38-73).                                                         */
+int sddmm_plan_create(const sddmm_coo *S, int32_t K, int32_t tile_size_x, int32_t tile_size_y,
+                      uint32_t flags, sddmm_plan **out);
+
+/* Same, for a CSR pattern that already lives in device memory (d_row_ptr:
+ * n_rows+1 int32, d_col_ind: nnz int32, sorted inside each row).  The plan
+ * borrows both arrays: they must outlive it.  The tiling pass runs from a
+ * host copy of the pattern made here.                                       */
+int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                             const int32_t *d_col_ind, int32_t K, int32_t tile_size_x,
+                             int32_t tile_size_y, uint32_t flags, sddmm_plan **out);
+
+int sddmm_plan_get_info(const sddmm_plan *plan, sddmm_plan_info *info);
+void sddmm_plan_destroy(sddmm_plan *plan);
+
+/* -------------------------------------------------------------- execute --- */
+
+/* Launches the SDDMM on `stream` (a hipStream_t, NULL = default stream) and
+ * returns without synchronising.  All four pointers are device pointers:
+ *   d_val  nnz fp32 in sorted order; NULL = the values uploaded with the plan
+ *          (for a plan made by sddmm_plan_create_device: NULL = no scaling,
+ *          out[p] = dot, the form the shipping reference kernel computes,
+ *          kernel.h:47-48)
+ *   d_W    n_rows*K, d_H  n_cols*K, row-major;  d_out  nnz fp32 (overwritten).
+ * Replaces the launch loop of sddmm_GPU, sddmm.cu:88-108, and
+ * comp_kernel_COO, kernel.h:2-52.                                           */
+int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                  float *d_out, void *stream);
+
+/* Host-pointer form with the calling convention of the reference's
+ * sddmm_GPU(S, tiledS, P, W, H) (sddmm.cu:32): copies W and H to the device,
+ * runs the kernels between two events, copies the result back into h_out
+ * (nnz fp32, sorted order) and reports the kernel-only time in milliseconds,
+ * the quantity the reference prints at sddmm.cu:109-114.                    */
+int sddmm_gpu(const sddmm_plan *plan, const float *h_W, const float *h_H, float *h_out,
+              float *kernel_ms);
+
+/* Number of visible devices and the gcnArchName of device 0 ("" if none). */
+int sddmm_device_info(int *n_devices, char *arch, int arch_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SDDMM_H */

@@ -1,0 +1,131 @@
+// sddmm -- command-line driver with the reference's calling convention
+// (README.md:21-33, HiPC18/src/sddmm.cu:247-286):
+//
+//     sddmm input K tile_size_X tile_size_Y [options]
+//
+// It prints the same three lines as the reference binary ("Matrix info",
+// "Tilesize", "Time for SDDMM with K = ...", sddmm.cu:267,282,114), runs with
+// the reference's dense factors (0.1*drand48(), util.h:75-81) and reports the
+// kernel-only time.  tile_size_X is the number of columns of S per LDS tile,
+// tile_size_Y the row-panel height (README's names for the 3rd and 4th
+// positional arguments; 0 = let the planner choose).
+#include <algorithm>
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+#include "../../include/sddmm.h"
+
+static void usage()
+{
+    fprintf(stderr,
+            "usage: sddmm input K tile_size_X tile_size_Y [options]\n"
+            "  input          Matrix Market coordinate file (or a .bin written by --save-bin)\n"
+            "  K              rank of W (rows x K) and H (cols x K)\n"
+            "  tile_size_X    columns of S per LDS tile (0 = auto)\n"
+            "  tile_size_Y    row-panel height (0 = auto)\n"
+            "options:\n"
+            "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
+            "  --kernel NAME  auto | row | lds\n"
+            "  --runs N       timed repetitions (default 1; the median is printed)\n"
+            "  --save-bin F   write the parsed, sorted matrix to F for fast re-loading\n"
+            "  --json         also print one JSON line with the plan and timing\n");
+}
+
+static bool ends_with(const std::string &s, const char *suf)
+{
+    size_t n = strlen(suf);
+    return s.size() >= n && s.compare(s.size() - n, n, suf) == 0;
+}
+
+#define CHECK(call)                                                        \
+    do {                                                                   \
+        int rc_ = (call);                                                  \
+        if (rc_ != SDDMM_OK) {                                             \
+            fprintf(stderr, "sddmm: %s\n", sddmm_last_error());            \
+            return 10 + rc_;                                               \
+        }                                                                  \
+    } while (0)
+
+int main(int argc, char **argv)
+{
+    if (argc < 5) {
+        usage();
+        return 2;
+    }
+    const std::string input = argv[1];
+    char *endp = nullptr;
+    long K = strtol(argv[2], &endp, 10);
+    if (*endp || K < 1) { fprintf(stderr, "sddmm: K must be a positive integer\n"); return 2; }
+    long tx = strtol(argv[3], &endp, 10);
+    if (*endp || tx < 0) { fprintf(stderr, "sddmm: tile_size_X must be a non-negative integer\n"); return 2; }
+    long ty = strtol(argv[4], &endp, 10);
+    if (*endp || ty < 0) { fprintf(stderr, "sddmm: tile_size_Y must be a non-negative integer\n"); return 2; }
+    bool transpose = false, json = false;
+    int runs = 1;
+    uint32_t kernel = SDDMM_KERNEL_AUTO;
+    std::string save_bin;
+    for (int i = 5; i < argc; ++i) {
+        std::string a = argv[i];
+        if (a == "--transpose") transpose = true;
+        else if (a == "--json") json = true;
+        else if (a == "--runs" && i + 1 < argc) runs = std::max(1, atoi(argv[++i]));
+        else if (a == "--save-bin" && i + 1 < argc) save_bin = argv[++i];
+        else if (a == "--kernel" && i + 1 < argc) {
+            std::string k = argv[++i];
+            if (k == "auto") kernel = SDDMM_KERNEL_AUTO;
+            else if (k == "row") kernel = SDDMM_KERNEL_ROW_GATHER;
+            else if (k == "lds") kernel = SDDMM_KERNEL_LDS_TILE;
+            else { fprintf(stderr, "sddmm: unknown kernel '%s'\n", k.c_str()); return 2; }
+        } else { usage(); return 2; }
+    }
+
+    auto t0 = std::chrono::steady_clock::now();
+    sddmm_coo *S = nullptr;
+    if (ends_with(input, ".bin")) CHECK(sddmm_read_bin(input.c_str(), &S));
+    else CHECK(sddmm_read_mtx(input.c_str(), &S));
+    int64_t n_rows, n_cols, nnz;
+    int sorted;
+    if (transpose) CHECK(sddmm_coo_transpose_sort(S));
+    CHECK(sddmm_coo_info(S, &n_rows, &n_cols, &nnz, &sorted));
+    printf("\nMatrix info:  rows: %lld, cols: %lld, nnz: %lld\n", (long long)n_rows, (long long)n_cols, (long long)nnz);
+    if (!sorted) {
+        fprintf(stderr, "sddmm: input is not row-sorted; sorting it\n");
+        CHECK(sddmm_coo_sort_rows(S));
+    }
+    if (!save_bin.empty()) CHECK(sddmm_write_bin(S, save_bin.c_str()));
+    double read_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+
+    sddmm_plan *plan = nullptr;
+    CHECK(sddmm_plan_create(S, (int32_t)K, (int32_t)tx, (int32_t)ty, kernel, &plan));
+    sddmm_plan_info info;
+    CHECK(sddmm_plan_get_info(plan, &info));
+    printf("\nTilesize: X = %d, tilesize: Y = %d, TB: %d\n", info.tile_size_x, info.tile_size_y, info.block);
+
+    std::vector<float> W((size_t)n_rows * K), H((size_t)n_cols * K), out((size_t)nnz);
+    CHECK(sddmm_init_reference(W.data(), n_rows, (int32_t)K));
+    CHECK(sddmm_init_reference(H.data(), n_cols, (int32_t)K));
+    std::vector<float> ms((size_t)runs);
+    for (int r = 0; r < runs; ++r) CHECK(sddmm_gpu(plan, W.data(), H.data(), out.data(), &ms[r]));
+    std::sort(ms.begin(), ms.end());
+    float med = ms[ms.size() / 2];
+    printf("\nTime for SDDMM with K = %ld : %g ms\n", K, med);
+    double sum = 0;
+    for (float v : out) sum += v;
+    if (json) {
+        double gflops = med > 0 ? 2.0 * (double)nnz * (double)K / (med * 1e6) : 0.0;
+        double balg = 12.0 * nnz + 4.0 * (n_rows + 1) + 4.0 * K * (double)(info.rows_touched + info.cols_touched);
+        printf("{\"rows\": %lld, \"cols\": %lld, \"nnz\": %lld, \"K\": %ld, \"tile_size_x\": %d, \"tile_size_y\": %d, "
+               "\"kernel\": %d, \"lanes_per_nnz\": %d, \"lds_bytes\": %d, \"grid\": %d, \"block\": %d, "
+               "\"n_col_tiles\": %d, \"read_ms\": %.3f, \"plan_ms\": %.3f, \"kernel_ms\": %.6f, \"gflops\": %.3f, "
+               "\"alg_gbps\": %.3f, \"checksum\": %.9g}\n",
+               (long long)n_rows, (long long)n_cols, (long long)nnz, K, info.tile_size_x, info.tile_size_y, info.kernel,
+               info.lanes_per_nnz, info.lds_bytes, info.grid, info.block, info.n_col_tiles, read_ms, info.plan_ms,
+               (double)med, gflops, med > 0 ? balg / (med * 1e6) : 0.0, sum);
+    }
+    sddmm_plan_destroy(plan);
+    sddmm_coo_destroy(S);
+    return 0;
+}
