@@ -1,0 +1,194 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real
+MI355X.  Pattern and output order are bit-exact by construction of the checks
+(outputs are compared position by position with the oracle's, which runs on
+the same sorted arrays); values must agree within 1e-5*sqrt(K) relative per
+nonzero (see conftest.parity_report for nonzeros that cancel to ~0)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import parity_report
+from sddmm_gpu_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE}
+
+
+def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_vals=True):
+    """d: dict from synth (CPU tensors).  Returns (out numpy, plan info)."""
+    dev = torch.device("cuda:0")
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], rows, cols, vals)
+    K = K or d["K"]
+    plan = S.plan(K, tile_x, tile_y, kernel)
+    W = d["W"].to(dev).contiguous(); H = d["H"].to(dev).contiguous()
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    dval = 0 if use_plan_vals else d["val"].to(dev)
+    plan.execute(0 if use_plan_vals else dval.data_ptr(), W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), plan.info()
+
+
+def check(d, out, oracle, K=None):
+    K = K or d["K"]
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    W = d["W"].numpy(); H = d["H"].numpy()
+    cpu = oracle.sddmm_csr(d["row_ptr"].numpy(), cols, vals, W, H)
+    assert np.array_equal(cpu, oracle.sddmm_coo(rows, cols, vals, W, H))
+    f64, absp = oracle.sddmm_f64(rows, cols, vals, W, H)
+    assert out.shape == cpu.shape and np.all(np.isfinite(out))
+    rep = parity_report(out, cpu, K, absp)
+    assert rep["violations"] == 0, rep
+    # the GPU's tree-shaped sum must not be less accurate than the sequential CPU sum
+    err_gpu = np.abs(out - f64).max(); err_cpu = np.abs(cpu - f64).max()
+    assert err_gpu <= 2 * err_cpu + 1e-30, (err_gpu, err_cpu)
+    return rep
+
+
+@pytest.mark.parametrize("kernel", ["row", "lds"])
+def test_config1_uniform_single_tile(oracle, kernel):
+    d = synth.make(1)
+    out, info = run_gpu(d, tile_x=4096, tile_y=4096, kernel=KERNELS[kernel])
+    rep = check(d, out, oracle)
+    assert info["nnz"] == d["nnz"] and info["K"] == 32
+    if kernel == "lds":
+        assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] <= 1280
+    print(rep)
+
+
+@pytest.mark.parametrize("kernel,tx,ty", [("auto", 192, 50000), ("row", 0, 0), ("lds", 64, 48)])
+def test_config2_bag_of_words(oracle, kernel, tx, ty):
+    d = synth.make(2)
+    out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=KERNELS.get(kernel, capi.KERNEL_AUTO))
+    rep = check(d, out, oracle)
+    if kernel == "auto":
+        assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] == 160  # 192 rows of K=256 exceed 160 KB
+    print(info, rep)
+
+
+@pytest.mark.parametrize("cfg,scale,K", [(3, 0.02, 128), (3, 0.02, 32), (3, 0.01, 256), (3, 0.005, 512),
+                                         (4, 2.0 ** -7, 64), (5, 2.0 ** -6, 512), (5, 2.0 ** -7, 1024)])
+@pytest.mark.parametrize("kernel", ["row", "lds"])
+def test_scaled_configs(oracle, cfg, scale, K, kernel):
+    d = synth.make(cfg, scale, K=K)
+    out, info = run_gpu(d, kernel=KERNELS[kernel])
+    check(d, out, oracle)
+
+
+@pytest.mark.parametrize("K", [1, 3, 4, 20, 36, 96, 100, 192, 384, 2048, 2052])
+def test_odd_ranks(oracle, K):
+    d = synth.uniform_random(300, 500, 0.05, K=K, seed=40 + K)
+    for kernel in ("row", "lds"):
+        out, info = run_gpu(d, tile_x=64, kernel=KERNELS[kernel])
+        check(d, out, oracle)
+
+
+def test_edge_shapes(oracle):
+    rng = np.random.default_rng(7)
+    K = 64
+    cases = {
+        "single_nonzero": ([5], [7]),
+        "one_full_row": (np.full(300, 3), np.arange(300)),
+        "one_full_col": (np.arange(200), np.full(200, 11)),
+        "diag": (np.arange(150), np.arange(150)),
+        "first_and_last": ([0, 299], [0, 299]),
+        "exactly_64": (np.repeat(np.arange(8), 8), np.tile(np.arange(8), 8)),
+        "exactly_65": (np.concatenate([np.repeat(np.arange(8), 8), [9]]), np.concatenate([np.tile(np.arange(8), 8), [0]])),
+    }
+    for name, (r, c) in cases.items():
+        r = np.asarray(r, np.int32); c = np.asarray(c, np.int32)
+        n, m = 300, 300
+        d = dict(n_rows=n, n_cols=m, nnz=len(r), K=K, row_ind=torch.from_numpy(r), col_ind=torch.from_numpy(c),
+                 row_ptr=torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(r, minlength=n))]).astype(np.int32)),
+                 val=torch.from_numpy(rng.standard_normal(len(r)).astype(np.float32)),
+                 W=torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32)),
+                 H=torch.from_numpy(rng.standard_normal((m, K)).astype(np.float32)))
+        for kernel, tx, ty in (("row", 0, 0), ("lds", 7, 3), ("lds", 300, 1)):
+            out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=KERNELS[kernel])
+            check(d, out, oracle)
+
+
+def test_empty_matrix_and_empty_rows(oracle):
+    S = capi.Coo.from_arrays(10, 10, [], [])
+    plan = S.plan(32)
+    plan.execute(0, 0, 0, 0)  # nnz == 0: nothing is touched
+    assert plan.info()["nnz"] == 0
+    d = synth.uniform_random(2000, 100, 0.002, K=32, seed=9)  # most rows empty
+    assert (np.diff(d["row_ptr"].numpy()) == 0).mean() > 0.5
+    for kernel in ("row", "lds"):
+        out, _ = run_gpu(d, tile_x=16, tile_y=5, kernel=KERNELS[kernel])
+        check(d, out, oracle)
+
+
+def test_closed_forms_on_gpu():
+    d = synth.make(1)
+    dev = torch.device("cuda:0")
+    for kernel in ("row", "lds"):
+        for K in (32, 100, 7):
+            S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+            plan = S.plan(K, 256, 64, KERNELS[kernel])
+            W = torch.ones(d["n_rows"], K, device=dev); H = torch.ones(d["n_cols"], K, device=dev)
+            out = torch.empty(d["nnz"], device=dev)
+            plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+            assert torch.equal(out.cpu(), d["val"] * K)            # W = H = 1  ->  K * val
+            j = torch.randint(0, K, (d["n_cols"],), generator=torch.Generator().manual_seed(1))
+            Hoh = torch.zeros(d["n_cols"], K); Hoh[torch.arange(d["n_cols"]), j] = 1.0
+            Wr = torch.randn(d["n_rows"], K, generator=torch.Generator().manual_seed(2))
+            Wd = Wr.to(dev); Hd = Hoh.to(dev)
+            plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+            expect = Wr[d["row_ind"].long(), j[d["col_ind"].long()]] * d["val"]
+            assert torch.equal(out.cpu(), expect)                  # one-hot H picks W[r, j(c)]
+
+
+def test_value_sources_and_host_form(oracle):
+    d = synth.make(3, 0.01, K=64)
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    W = d["W"].numpy(); H = d["H"].numpy()
+    dev = torch.device("cuda:0")
+    # (a) values passed at execute override the plan's
+    out_a, _ = run_gpu(d, use_plan_vals=False)
+    check(d, out_a, oracle)
+    # (b) a plan over a device-resident CSR, no values: out = dot (the shipping reference's form)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
+    for kernel in (capi.KERNEL_ROW_GATHER, capi.KERNEL_LDS_TILE):
+        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, 128, 32,
+                                         kernel, keep=(rp, ci))
+        Wd = d["W"].to(dev); Hd = d["H"].to(dev); out = torch.empty(d["nnz"], device=dev)
+        plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+        cpu = oracle.sddmm_coo(rows, cols, vals, W, H, apply_val=False)
+        _, absp = oracle.sddmm_f64(rows, cols, np.ones_like(vals), W, H)
+        assert parity_report(out.cpu().numpy(), cpu, 64, absp)["violations"] == 0
+        dv = d["val"].to(dev)
+        plan.execute(dv.data_ptr(), Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+        check(d, out.cpu().numpy(), oracle)
+    # (c) host-pointer form with the reference's sddmm_GPU convention
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], rows, cols, vals)
+    out_c, ms = S.plan(64).gpu(W, H)
+    check(d, out_c, oracle)
+    assert ms > 0
+
+
+def test_device_plan_rejects_bad_csr():
+    dev = torch.device("cuda:0")
+    rp = torch.tensor([0, 2, 3], dtype=torch.int32, device=dev)
+    bad_sorted = torch.tensor([5, 1, 0], dtype=torch.int32, device=dev)
+    with pytest.raises(capi.SddmmError) as e:
+        capi.Plan.from_device_csr(2, 8, 3, rp.data_ptr(), bad_sorted.data_ptr(), 32)
+    assert e.value.code == capi.ERR_UNSORTED
+    bad_range = torch.tensor([1, 9, 0], dtype=torch.int32, device=dev)
+    with pytest.raises(capi.SddmmError) as e:
+        capi.Plan.from_device_csr(2, 8, 3, rp.data_ptr(), bad_range.data_ptr(), 32)
+    assert e.value.code == capi.ERR_RANGE
+
+
+def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
+    d = synth.make(2)
+    base, _ = run_gpu(d, kernel=capi.KERNEL_ROW_GATHER)
+    d2 = dict(d); d2["W"] = d["W"] * 4.0
+    out4, _ = run_gpu(d2, kernel=capi.KERNEL_ROW_GATHER)
+    assert np.array_equal(out4, base * 4.0)
+    _, absp = oracle.sddmm_f64(d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy(), d["W"].numpy(), d["H"].numpy())
+    for tx, ty in ((160, 50000), (50, 10), (1, 1), (12419, 1500)):
+        out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=capi.KERNEL_LDS_TILE)
+        assert parity_report(out, base, d["K"], absp)["violations"] == 0, (tx, ty)
