@@ -82,7 +82,7 @@ def main():
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--K", type=int, default=None)
-    ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds"])
+    ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds", "panel"])
     ap.add_argument("--tile-x", type=int, default=0)
     ap.add_argument("--tile-y", type=int, default=0)
     ap.add_argument("--sweep-k", action="store_true", help="also report K = 32, 128, 256, 512")
@@ -99,7 +99,7 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE}[args.kernel]
+    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}[args.kernel]
     names = {1: "uniform 4096^2 1%", 2: "bag-of-words 1500x12419", 3: "recommender 480189x17770 ~100M nnz",
              4: "R-MAT 2^22 ~200M nnz", 5: "banded 2^20 64/row"}
 
@@ -151,7 +151,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": names[args.config] + (f" (scale {args.scale})" if args.scale != 1.0 else ""),
                    "n_rows": d["n_rows"], "n_cols": d["n_cols"], "nnz": d["nnz"], "K": K0, "seed": d["seed"],
-                   "kernel": {1: "row_gather", 2: "lds_tile"}[info["kernel"]],
+                   "kernel": {1: "row_gather", 2: "lds_tile", 3: "panel"}[info["kernel"]],
                    "tile_size_x": info["tile_size_x"], "tile_size_y": info["tile_size_y"],
                    "lanes_per_nnz": info["lanes_per_nnz"], "grid": info["grid"], "block": info["block"],
                    "lds_bytes": info["lds_bytes"], "plan_ms": round(info["plan_ms"], 1)},

@@ -41,7 +41,8 @@ enum {
 enum {
     SDDMM_KERNEL_AUTO = 0,
     SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM */
-    SDDMM_KERNEL_LDS_TILE = 2    /* column tiles of H staged in LDS, W row in VGPRs */
+    SDDMM_KERNEL_LDS_TILE = 2,   /* column tiles of H staged in LDS, W row (re)loaded per row run */
+    SDDMM_KERNEL_PANEL = 3       /* row panels of W resident in VGPRs, column tiles of H swept through LDS */
 };
 
 typedef struct sddmm_coo sddmm_coo;   /* host-side sparse matrix (COO, int32/int32/fp32) */

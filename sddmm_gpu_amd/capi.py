@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsddmm_hip.so")
 
 OK, ERR_ARG, ERR_IO, ERR_FORMAT, ERR_RANGE, ERR_UNSORTED, ERR_HIP, ERR_NOMEM = range(8)
-KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE = 0, 1, 2
+KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL = 0, 1, 2, 3
 
 
 class SddmmError(RuntimeError):

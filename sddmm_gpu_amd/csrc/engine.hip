@@ -1,299 +1,15 @@
-// Device side of the SDDMM engine for gfx950 (MI355X): plan construction
-// (stream descriptors for the kernels, upload) and the HIP kernels.
-//
-// Both kernel families walk a "stream" of nonzeros in batches of 64 (one per
-// lane of a wavefront):
-//   row-gather : the stream is the sorted S itself, cut into fixed chunks;
-//   LDS-tile   : the stream is S in tile order (column tile by column tile,
-//                rows ascending inside a tile) reached through the permutation
-//                the tiling pass produced; the workgroup stages the tile's H
-//                rows in LDS first.
-// A batch loads its 64 column indices / values / outputs coalesced.  The rows
-// of the 64 nonzeros come from two small side arrays (first segment of the
-// batch + a 64-bit mask of "a new row starts here"), so no per-nonzero row
-// index is read.  Inside a batch, groups of G lanes each take G consecutive
-// nonzeros: for each, the group reads the H row (from LDS or global) as
-// contiguous 16-byte pieces, multiplies with the W row slice it keeps in
-// VGPRs while the row lasts, and the G partial sums of G nonzeros are reduced
-// together by a butterfly of cross-lane exchanges that leaves nonzero i's dot
-// product in lane i, which scales it by S.val and stores it.
+// Plan construction (stream descriptors for the kernels, upload) and launch
+// of the SDDMM engine for gfx950 (MI355X).
 #include <hip/hip_runtime.h>
 #include <chrono>
 #include <cstring>
 #include <new>
 #include "internal.hpp"
+#include "kernels.hpp"
 
 using namespace sddmm;
 
 namespace {
-
-struct WorkItem {
-    int32_t begin, end;   // stream positions
-    int32_t batch_base;   // index of the item's first batch in batch_seg / batch_mask
-    int32_t tile;         // column tile staged in LDS (-1: none)
-};
-
-struct KArgs {
-    const int32_t *col_ind;    // [nnz] sorted order
-    const float *val;          // [nnz] or null (no scaling)
-    const float *W, *H;
-    float *out;
-    const int32_t *perm;       // stream position -> sorted position, null = identity
-    const int32_t *seg_row;    // segment -> global row, null = identity
-    const int32_t *batch_seg;  // per batch: segment of its first nonzero
-    const uint64_t *batch_mask;  // per batch: bit L (L >= 1) set if lane L starts a new segment
-    const WorkItem *items;     // null: fixed chunks of `chunk` nonzeros over [0, nnz)
-    int32_t n_items;
-    int32_t nnz;
-    int32_t chunk;
-    int32_t K;
-    int32_t tile_x;
-    int32_t n_cols;
-};
-
-constexpr int kRowGatherBlock = 256;   // 4 waves
-constexpr int kRowGatherBatchesPerWave = 8;
-constexpr int kLdsBlock = 1024;        // 16 waves, one workgroup per CU
-constexpr int kLdsMaxBytes = 160 * 1024;
-
-__device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float acc)
-{
-    acc = fmaf(a.x, b.x, acc);
-    acc = fmaf(a.y, b.y, acc);
-    acc = fmaf(a.z, b.z, acc);
-    acc = fmaf(a.w, b.w, acc);
-    return acc;
-}
-
-// Reduces G accumulators across the G lanes of a group so that lane i of the
-// group ends with the full sum of accumulator i (returned).
-template <int G>
-__device__ __forceinline__ float transpose_reduce(float (&acc)[G], int l)
-{
-#pragma unroll
-    for (int s = G / 2; s >= 1; s >>= 1) {
-        const bool upper = (l & s) != 0;
-#pragma unroll
-        for (int j = 0; j < s; ++j) {
-            float keep = upper ? acc[j + s] : acc[j];
-            float send = upper ? acc[j] : acc[j + s];
-            acc[j] = keep + __shfl_xor(send, s, G);
-        }
-    }
-    return acc[0];
-}
-
-// K = 4 * (number of float4 per row); each lane of a group owns KPL float4
-// slots of a row: slot j sits at float4 index (((j + rot) % KPL) * G + l).  `rot`
-// differs between the groups that share one 16-lane LDS access phase, so that
-// their 16-byte reads fall into different banks when rows are a multiple of
-// 256 bytes apart.  EXACT: K == 4*G*KPL (no slot is out of range).
-template <int G, int KPL, bool EXACT, bool LDS_TILE>
-__global__ __launch_bounds__(LDS_TILE ? kLdsBlock : kRowGatherBlock)
-void sddmm_stream_kernel(const KArgs a)
-{
-    extern __shared__ float4 lds_tile[];
-    constexpr int NW = (LDS_TILE ? kLdsBlock : kRowGatherBlock) / 64;
-    constexpr int PHASE_GROUPS = (16 / G) >= 1 ? (16 / G) : 1;
-    constexpr int ROT_MASK = (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL) - 1;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int l = lane & (G - 1);
-    const int rot = (lane / G) & ROT_MASK;
-    const int K4 = a.K >> 2;
-
-    int slot[KPL];
-#pragma unroll
-    for (int j = 0; j < KPL; ++j) slot[j] = (((j + rot) % KPL) * G + l);
-
-    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W);
-    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H);
-
-    int item0, item1;
-    if (LDS_TILE) {  // contiguous run of items per workgroup: the tile changes rarely
-        item0 = (int)((int64_t)a.n_items * blockIdx.x / gridDim.x);
-        item1 = (int)((int64_t)a.n_items * (blockIdx.x + 1) / gridDim.x);
-    } else {
-        item0 = blockIdx.x;
-        item1 = item0 + 1;
-    }
-    int cur_tile = -1;
-    int tile_base = 0;
-
-    for (int it = item0; it < item1; ++it) {
-        int begin, end, batch_base;
-        if (LDS_TILE) {
-            const WorkItem wi = a.items[it];
-            begin = wi.begin; end = wi.end; batch_base = wi.batch_base;
-            if (wi.tile != cur_tile) {
-                __syncthreads();  // everyone is done with the previous tile
-                cur_tile = wi.tile;
-                tile_base = cur_tile * a.tile_x;
-                int rows = min(a.tile_x, a.n_cols - tile_base);
-                const float4 *src = H4 + (size_t)tile_base * K4;
-                const int n4 = rows * K4;
-                for (int i = threadIdx.x; i < n4; i += blockDim.x) lds_tile[i] = src[i];
-                __syncthreads();
-            }
-        } else {
-            begin = it * a.chunk;
-            end = min(a.nnz, begin + a.chunk);
-            batch_base = begin >> 6;
-        }
-        const int nb = (end - begin + 63) >> 6;
-        const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
-
-        int cur_row = -1;
-        float4 w[KPL];
-#pragma unroll
-        for (int j = 0; j < KPL; ++j) w[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-
-        for (int bi = b0; bi < b1; ++bi) {
-            const int pos = begin + (bi << 6) + lane;
-            const bool valid = pos < end;
-            const int gb = batch_base + bi;
-            const int seg0 = a.batch_seg[gb];
-            const uint64_t mask = a.batch_mask[gb];
-            const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
-            const int seg = seg0 + __popcll(mask & le);
-            int row = -1, p = 0, col = 0;
-            float v = 0.f;
-            if (valid) {
-                row = a.seg_row ? a.seg_row[seg] : seg;
-                p = a.perm ? a.perm[pos] : pos;
-                col = a.col_ind[p];
-                v = a.val ? a.val[p] : 1.0f;
-            }
-            float acc[G];
-#pragma unroll
-            for (int i = 0; i < G; ++i) acc[i] = 0.f;
-
-            const int row_first = __shfl(row, 0, G);
-            const int row_last = __shfl(row, G - 1, G);
-            if (row_first == row_last && row_last >= 0) {
-                // all G nonzeros of this group lie in one row: no checks inside
-                if (row_first != cur_row) {
-                    cur_row = row_first;
-                    const float4 *wr = W4 + (size_t)cur_row * K4;
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j)
-                        w[j] = (EXACT || slot[j] < K4) ? wr[slot[j]] : make_float4(0.f, 0.f, 0.f, 0.f);
-                }
-#pragma unroll
-                for (int i = 0; i < G; ++i) {
-                    const int c_i = __shfl(col, i, G);
-                    const float4 *hr = LDS_TILE ? (lds_tile + (size_t)(c_i - tile_base) * K4)
-                                                : (H4 + (size_t)c_i * K4);
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j)
-                        if (EXACT || slot[j] < K4) acc[i] = dot4(w[j], hr[slot[j]], acc[i]);
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < G; ++i) {
-                    const int r_i = __shfl(row, i, G);
-                    const int c_i = __shfl(col, i, G);
-                    if (r_i >= 0) {
-                        if (r_i != cur_row) {
-                            cur_row = r_i;
-                            const float4 *wr = W4 + (size_t)cur_row * K4;
-#pragma unroll
-                            for (int j = 0; j < KPL; ++j)
-                                w[j] = (EXACT || slot[j] < K4) ? wr[slot[j]] : make_float4(0.f, 0.f, 0.f, 0.f);
-                        }
-                        const float4 *hr = LDS_TILE ? (lds_tile + (size_t)(c_i - tile_base) * K4)
-                                                    : (H4 + (size_t)c_i * K4);
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j)
-                            if (EXACT || slot[j] < K4) acc[i] = dot4(w[j], hr[slot[j]], acc[i]);
-                    }
-                }
-            }
-            const float sum = transpose_reduce<G>(acc, l);
-            if (valid) a.out[p] = sum * v;
-        }
-    }
-}
-
-// Any K >= 1: 8 lanes per nonzero striding over the row one float at a time,
-// W re-read through the cache.  The slow, always-correct path.
-__global__ __launch_bounds__(kRowGatherBlock)
-void sddmm_generic_kernel(const KArgs a)
-{
-    constexpr int G = 8;
-    constexpr int NW = kRowGatherBlock / 64;
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int l = lane & (G - 1);
-    const int begin = blockIdx.x * a.chunk;
-    const int end = min(a.nnz, begin + a.chunk);
-    const int batch_base = begin >> 6;
-    const int nb = (end - begin + 63) >> 6;
-    const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
-    for (int bi = b0; bi < b1; ++bi) {
-        const int pos = begin + (bi << 6) + lane;
-        const bool valid = pos < end;
-        const int gb = batch_base + bi;
-        const uint64_t mask = a.batch_mask[gb];
-        const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
-        const int seg = a.batch_seg[gb] + __popcll(mask & le);
-        int row = -1, col = 0;
-        float v = 0.f;
-        if (valid) {
-            row = a.seg_row ? a.seg_row[seg] : seg;
-            col = a.col_ind[pos];
-            v = a.val ? a.val[pos] : 1.0f;
-        }
-        float acc[G];
-#pragma unroll
-        for (int i = 0; i < G; ++i) {
-            const int r_i = __shfl(row, i, G);
-            const int c_i = __shfl(col, i, G);
-            float s = 0.f;
-            if (r_i >= 0) {
-                const float *wr = a.W + (size_t)r_i * a.K;
-                const float *hr = a.H + (size_t)c_i * a.K;
-                for (int t = l; t < a.K; t += G) s = fmaf(wr[t], hr[t], s);
-            }
-            acc[i] = s;
-        }
-        const float sum = transpose_reduce<G>(acc, l);
-        if (valid) a.out[pos] = sum * v;
-    }
-}
-
-struct Variant {
-    int G, KPL;
-    bool exact;
-};
-
-// lanes per nonzero and float4 slots per lane for a given K (K % 4 == 0)
-Variant pick_variant(int K)
-{
-    const int K4 = K / 4;
-    const int cand[][2] = {{8, 1}, {8, 2}, {8, 3}, {8, 4}, {8, 6}, {8, 8}, {16, 6}, {16, 8}, {32, 6}, {32, 8}, {64, 6}, {64, 8}};
-    for (auto &c : cand)
-        if (c[0] * c[1] == K4) return {c[0], c[1], true};
-    for (auto &c : cand)
-        if (c[0] * c[1] >= K4) return {c[0], c[1], false};
-    return {0, 0, false};  // K > 2048: generic kernel
-}
-
-using KernelFn = void (*)(const KArgs);
-
-template <bool LDS_TILE>
-KernelFn lookup(const Variant &v)
-{
-#define SDDMM_CASE(g, kpl)                                                              \
-    if (v.G == g && v.KPL == kpl)                                                       \
-        return v.exact ? (KernelFn)sddmm_stream_kernel<g, kpl, true, LDS_TILE>          \
-                       : (KernelFn)sddmm_stream_kernel<g, kpl, false, LDS_TILE>;
-    SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 3) SDDMM_CASE(8, 4) SDDMM_CASE(8, 6) SDDMM_CASE(8, 8)
-    SDDMM_CASE(16, 6) SDDMM_CASE(16, 8) SDDMM_CASE(32, 6) SDDMM_CASE(32, 8) SDDMM_CASE(64, 6) SDDMM_CASE(64, 8)
-#undef SDDMM_CASE
-    return nullptr;
-}
 
 #define HIP_TRY(expr)                                                                               \
     do {                                                                                            \
@@ -327,8 +43,17 @@ struct sddmm_plan {
     WorkItem *d_items = nullptr;
     int32_t n_items = 0;
     int32_t chunk = 0;
+    // panel kernel
+    PanelFn panel_fn = nullptr;
+    const int32_t *d_row_ptr = nullptr;
+    bool own_row_ptr = false;
+    int32_t *d_slot_row = nullptr, *d_panel_tiles = nullptr;
+    int32_t n_panels = 0;
     ~sddmm_plan()
     {
+        if (own_row_ptr && d_row_ptr) (void)hipFree((void *)d_row_ptr);
+        if (d_slot_row) (void)hipFree(d_slot_row);
+        if (d_panel_tiles) (void)hipFree(d_panel_tiles);
         if (own_col && d_col) (void)hipFree((void *)d_col);
         if (d_val) (void)hipFree(d_val);
         if (d_perm) (void)hipFree(d_perm);
@@ -404,7 +129,7 @@ int device_ok()
 // Common plan builder from host CSR arrays.  d_col_borrowed != null: the
 // device already holds col_ind.
 int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr, const int32_t *col_ind,
-              const float *vals, const int32_t *d_col_borrowed, int32_t K, int32_t tile_x, int32_t tile_y,
+              const float *vals, const int32_t *d_row_ptr_borrowed, const int32_t *d_col_borrowed, int32_t K, int32_t tile_x, int32_t tile_y,
               uint32_t flags, sddmm_plan **out)
 {
     auto t0 = std::chrono::steady_clock::now();
@@ -416,7 +141,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         return fail(SDDMM_ERR_RANGE, "plan: dense factor too large");
     if (int rc = device_ok()) return rc;
     int want = (int)(flags & 0xff);
-    if (want > SDDMM_KERNEL_LDS_TILE) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
+    if (want > SDDMM_KERNEL_PANEL) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
 
     sddmm_plan *P = new (std::nothrow) sddmm_plan;
     if (!P) return fail(SDDMM_ERR_NOMEM, "plan: out of memory");
@@ -436,6 +161,9 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     if (kernel == SDDMM_KERNEL_AUTO)
         kernel = (have_fast && tile_x > 0 && tile_x < n_cols && fit_x >= 8) ? SDDMM_KERNEL_LDS_TILE : SDDMM_KERNEL_ROW_GATHER;
     if (kernel == SDDMM_KERNEL_LDS_TILE && (!have_fast || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
+    // the panel kernel works on K slices of 128, 64 or 32 elements
+    const int ks = (K % 128 == 0) ? 128 : (K % 64 == 0) ? 64 : (K % 32 == 0) ? 32 : 0;
+    if (kernel == SDDMM_KERNEL_PANEL && ks == 0) kernel = SDDMM_KERNEL_ROW_GATHER;
     I.kernel = kernel;
     I.lanes_per_nnz = have_fast ? var.G : 8;
     P->variant = var;
@@ -460,6 +188,77 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
 
     std::vector<int32_t> batch_seg;
     std::vector<uint64_t> batch_mask;
+    if (kernel == SDDMM_KERNEL_PANEL) {
+        const PanelVariant pv = pick_panel_variant(ks);
+        P->panel_fn = panel_kernel(pv);
+        if (!P->panel_fn) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", ks);
+        const int32_t fit = kLdsMaxBytes / (ks * 4);
+        int32_t x = tile_x > 0 ? std::min(tile_x, fit) : fit;
+        x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
+        const int octs_cap = pv.S * pv.NWAVES;  // octets (8 rows, one per lane group of a wave) per panel
+        int octs = octs_cap;
+        if (tile_y > 0) octs = (int)std::max<int64_t>(1, std::min<int64_t>(octs_cap, ((int64_t)tile_y + 7) / 8));
+        const int rows_per_panel = octs * 8;
+        // panels: contiguous runs of non-empty rows (keeps the column locality of
+        // neighbouring rows); inside a panel rows are ranked by length so that the
+        // 8 groups of a wave work on rows of similar length in the same slot
+        std::vector<int32_t> ne;
+        ne.reserve((size_t)I.rows_touched);
+        for (int64_t r = 0; r < n_rows; ++r)
+            if (row_ptr[r + 1] > row_ptr[r]) ne.push_back((int32_t)r);
+        const int64_t n_panels = ((int64_t)ne.size() + rows_per_panel - 1) / rows_per_panel;
+        std::vector<int32_t> slot_row((size_t)n_panels * pv.S * pv.NWAVES * 8, -1);
+        std::vector<int32_t> panel_tiles((size_t)n_panels * 2, 0);
+        parallel_ranges(n_panels, 4, [&](int64_t pb, int64_t pe, int) {
+            std::vector<int32_t> rk;
+            for (int64_t p = pb; p < pe; ++p) {
+                const int64_t b = p * rows_per_panel, e = std::min<int64_t>(b + rows_per_panel, (int64_t)ne.size());
+                rk.assign(ne.begin() + b, ne.begin() + e);
+                std::stable_sort(rk.begin(), rk.end(), [&](int32_t u, int32_t v) {
+                    return row_ptr[u + 1] - row_ptr[u] > row_ptr[v + 1] - row_ptr[v];
+                });
+                int32_t cmin = INT32_MAX, cmax = 0;
+                for (size_t i = 0; i < rk.size(); ++i) {
+                    const int oct = (int)(i / 8), g = (int)(i % 8);
+                    const int slot = oct / pv.NWAVES, wave = oct % pv.NWAVES;
+                    slot_row[((((size_t)p * pv.S + slot) * pv.NWAVES) + wave) * 8 + g] = rk[i];
+                    cmin = std::min(cmin, col_ind[row_ptr[rk[i]]]);
+                    cmax = std::max(cmax, col_ind[row_ptr[rk[i] + 1] - 1]);
+                }
+                panel_tiles[2 * p] = cmin / x;
+                panel_tiles[2 * p + 1] = cmax / x;
+            }
+        });
+        if (d_row_ptr_borrowed) {
+            P->d_row_ptr = d_row_ptr_borrowed;
+        } else {
+            int32_t *d = nullptr;
+            HIP_TRY(hipMalloc((void **)&d, (size_t)(n_rows + 1) * 4));
+            HIP_TRY(hipMemcpy(d, row_ptr, (size_t)(n_rows + 1) * 4, hipMemcpyHostToDevice));
+            dev_bytes += (n_rows + 1) * 4;
+            P->d_row_ptr = d; P->own_row_ptr = true;
+        }
+        if (int rc = upload(&P->d_slot_row, slot_row, &dev_bytes)) return rc;
+        if (int rc = upload(&P->d_panel_tiles, panel_tiles, &dev_bytes)) return rc;
+        P->n_panels = (int32_t)n_panels;
+        hipDeviceProp_t prop;
+        HIP_TRY(hipGetDeviceProperties(&prop, 0));
+        const int cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        I.tile_size_x = x; I.tile_size_y = rows_per_panel; I.k_slice = ks;
+        I.n_col_tiles = (int32_t)((n_cols + x - 1) / x); I.n_row_panels = (int32_t)n_panels;
+        I.n_blocks = 0;
+        for (int64_t p = 0; p < n_panels; ++p) I.n_blocks += panel_tiles[2 * p + 1] - panel_tiles[2 * p] + 1;
+        I.lanes_per_nnz = 8;
+        I.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>(cus, n_panels));
+        I.block = pv.NWAVES * 64;
+        I.lds_bytes = x * ks * 4;
+        HIP_TRY(hipFuncSetAttribute((const void *)P->panel_fn, hipFuncAttributeMaxDynamicSharedMemorySize, I.lds_bytes));
+        I.device_bytes = dev_bytes;
+        I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        guard.p = nullptr;
+        *out = P;
+        return SDDMM_OK;
+    }
     if (kernel == SDDMM_KERNEL_ROW_GATHER) {
         // segments = non-empty rows
         std::vector<int32_t> seg_end, seg_row;
@@ -475,7 +274,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1;
         I.grid = (int32_t)((nnz + P->chunk - 1) / P->chunk);
         I.block = kRowGatherBlock; I.lds_bytes = 0;
-        P->fn = have_fast ? lookup<false>(var) : (KernelFn)sddmm_generic_kernel;
+        P->fn = have_fast ? stream_kernel(var, false) : generic_kernel();
     } else {
         int32_t x = tile_x > 0 ? tile_x : fit_x;
         x = std::min(x, fit_x);
@@ -516,7 +315,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         I.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)cus, (int64_t)items.size()));
         I.block = kLdsBlock;
         I.lds_bytes = (int32_t)((int64_t)x * row_bytes);
-        P->fn = lookup<true>(var);
+        P->fn = stream_kernel(var, true);
         HIP_TRY(hipFuncSetAttribute((const void *)P->fn, hipFuncAttributeMaxDynamicSharedMemorySize, I.lds_bytes));
     }
     if (!P->fn) return fail(SDDMM_ERR_ARG, "plan: no kernel for K = %d", K);
@@ -543,7 +342,7 @@ int sddmm_plan_create(const sddmm_coo *S, int32_t K, int32_t tile_size_x, int32_
     try {
         std::vector<int32_t> rp;
         build_row_ptr(*S, rp);
-        return make_plan(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), S->vals.data(), nullptr, K,
+        return make_plan(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), S->vals.data(), nullptr, nullptr, K,
                          tile_size_x, tile_size_y, flags, out);
     } catch (const std::bad_alloc &) {
         return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create: out of host memory");
@@ -582,7 +381,7 @@ int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const 
             if (c == 2) return fail(SDDMM_ERR_RANGE, "sddmm_plan_create_device: a column index lies outside the matrix");
             if (c == 3) return fail(SDDMM_ERR_UNSORTED, "sddmm_plan_create_device: columns are not sorted inside a row");
         }
-        return make_plan(n_rows, n_cols, nnz, rp.data(), ci.data(), nullptr, d_col_ind, K, tile_size_x, tile_size_y,
+        return make_plan(n_rows, n_cols, nnz, rp.data(), ci.data(), nullptr, d_row_ptr, d_col_ind, K, tile_size_x, tile_size_y,
                          flags, out);
     } catch (const std::bad_alloc &) {
         return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create_device: out of host memory");
@@ -606,8 +405,24 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
     if (I.nnz == 0) return SDDMM_OK;
     if (!d_W || !d_H || !d_out) return fail(SDDMM_ERR_ARG, "sddmm_execute: NULL device pointer");
     if (((uintptr_t)d_W | (uintptr_t)d_H) & 15u)
-        if (I.K % 4 == 0 && plan->variant.G)
+        if (I.K % 4 == 0 && (plan->variant.G || I.kernel == SDDMM_KERNEL_PANEL))
             return fail(SDDMM_ERR_ARG, "sddmm_execute: W and H must be 16-byte aligned");
+    if (I.kernel == SDDMM_KERNEL_PANEL) {
+        PanelArgs pa{};
+        pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
+        pa.val = d_val ? d_val : plan->d_val;
+        pa.W = d_W; pa.H = d_H; pa.out = d_out;
+        pa.slot_row = plan->d_slot_row; pa.panel_tiles = plan->d_panel_tiles;
+        pa.n_panels = plan->n_panels; pa.tile_x = I.tile_size_x; pa.n_cols = (int32_t)I.n_cols; pa.K = I.K;
+        for (int k_off = 0; k_off < I.K; k_off += I.k_slice) {
+            pa.k_off = k_off;
+            pa.accumulate = k_off > 0;
+            hipLaunchKernelGGL(plan->panel_fn, dim3((unsigned)I.grid), dim3((unsigned)I.block), (size_t)I.lds_bytes,
+                               (hipStream_t)stream, pa);
+        }
+        HIP_TRY(hipGetLastError());
+        return SDDMM_OK;
+    }
     KArgs a{};
     a.col_ind = plan->d_col;
     a.val = d_val ? d_val : plan->d_val;

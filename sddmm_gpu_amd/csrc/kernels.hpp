@@ -1,0 +1,69 @@
+// Argument blocks and lookup functions shared by the plan builder (engine.hip)
+// and the kernel translation units.
+#pragma once
+#include <cstdint>
+
+namespace sddmm {
+
+struct WorkItem {
+    int32_t begin, end;   // stream positions
+    int32_t batch_base;   // index of the item's first batch in batch_seg / batch_mask
+    int32_t tile;         // column tile staged in LDS (-1: none)
+};
+
+struct KArgs {
+    const int32_t *col_ind;    // [nnz] sorted order
+    const float *val;          // [nnz] or null (no scaling)
+    const float *W, *H;
+    float *out;
+    const int32_t *perm;       // stream position -> sorted position, null = identity
+    const int32_t *seg_row;    // segment -> global row, null = identity
+    const int32_t *batch_seg;  // per batch: segment of its first nonzero
+    const uint64_t *batch_mask;  // per batch: bit L (L >= 1) set if lane L starts a new segment
+    const WorkItem *items;     // null: fixed chunks of `chunk` nonzeros over [0, nnz)
+    int32_t n_items;
+    int32_t nnz;
+    int32_t chunk;
+    int32_t K;
+    int32_t tile_x;
+    int32_t n_cols;
+};
+
+constexpr int kRowGatherBlock = 256;   // 4 waves
+constexpr int kRowGatherBatchesPerWave = 8;
+constexpr int kLdsBlock = 1024;        // 16 waves, one workgroup per CU
+constexpr int kLdsMaxBytes = 160 * 1024;
+
+struct Variant {
+    int G, KPL;   // lanes per nonzero, float4 slots per lane
+    bool exact;   // K == 4*G*KPL
+};
+using KernelFn = void (*)(const KArgs);
+
+// Panel kernel: rows of W resident in VGPRs, column tiles of H in LDS.
+struct PanelArgs {
+    const int32_t *row_ptr;   // [n_rows+1]
+    const int32_t *col_ind;   // [nnz] sorted order
+    const float *val;         // [nnz] or null (no scaling)
+    const float *W, *H;
+    float *out;
+    const int32_t *slot_row;  // [n_panels][S][NWAVES][8] row of each (slot, wave, group); -1 = none
+    const int32_t *panel_tiles;  // [n_panels][2] first and last column tile the panel touches
+    int32_t n_panels, tile_x, n_cols;
+    int32_t K;                // row length of W and H
+    int32_t k_off;            // first K element covered by this pass
+    int32_t accumulate;       // add to out instead of overwriting it
+};
+struct PanelVariant {
+    int KPL, S, NWAVES;       // float4 per lane (K slice = 32*KPL), row slots per 8-lane group, waves per workgroup
+};
+using PanelFn = void (*)(const PanelArgs);
+PanelVariant pick_panel_variant(int k_slice);
+PanelFn panel_kernel(const PanelVariant &v);
+
+// lanes per nonzero and float4 slots per lane for a given K (K % 4 == 0); G == 0: none
+Variant pick_variant(int K);
+KernelFn stream_kernel(const Variant &v, bool lds_tile);
+KernelFn generic_kernel();
+
+}  // namespace sddmm

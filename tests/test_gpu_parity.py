@@ -12,7 +12,7 @@ from sddmm_gpu_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
 
-KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE}
+KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}
 
 
 def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_vals=True):
@@ -46,7 +46,7 @@ def check(d, out, oracle, K=None):
     return rep
 
 
-@pytest.mark.parametrize("kernel", ["row", "lds"])
+@pytest.mark.parametrize("kernel", ["row", "lds", "panel"])
 def test_config1_uniform_single_tile(oracle, kernel):
     d = synth.make(1)
     out, info = run_gpu(d, tile_x=4096, tile_y=4096, kernel=KERNELS[kernel])
@@ -54,10 +54,12 @@ def test_config1_uniform_single_tile(oracle, kernel):
     assert info["nnz"] == d["nnz"] and info["K"] == 32
     if kernel == "lds":
         assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] <= 1280
+    if kernel == "panel":
+        assert info["kernel"] == capi.KERNEL_PANEL and info["k_slice"] == 32
     print(rep)
 
 
-@pytest.mark.parametrize("kernel,tx,ty", [("auto", 192, 50000), ("row", 0, 0), ("lds", 64, 48)])
+@pytest.mark.parametrize("kernel,tx,ty", [("auto", 192, 50000), ("row", 0, 0), ("lds", 64, 48), ("panel", 192, 50000), ("panel", 50, 100)])
 def test_config2_bag_of_words(oracle, kernel, tx, ty):
     d = synth.make(2)
     out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=KERNELS.get(kernel, capi.KERNEL_AUTO))
@@ -69,7 +71,7 @@ def test_config2_bag_of_words(oracle, kernel, tx, ty):
 
 @pytest.mark.parametrize("cfg,scale,K", [(3, 0.02, 128), (3, 0.02, 32), (3, 0.01, 256), (3, 0.005, 512),
                                          (4, 2.0 ** -7, 64), (5, 2.0 ** -6, 512), (5, 2.0 ** -7, 1024)])
-@pytest.mark.parametrize("kernel", ["row", "lds"])
+@pytest.mark.parametrize("kernel", ["row", "lds", "panel"])
 def test_scaled_configs(oracle, cfg, scale, K, kernel):
     d = synth.make(cfg, scale, K=K)
     out, info = run_gpu(d, kernel=KERNELS[kernel])
@@ -79,9 +81,11 @@ def test_scaled_configs(oracle, cfg, scale, K, kernel):
 @pytest.mark.parametrize("K", [1, 3, 4, 20, 36, 96, 100, 192, 384, 2048, 2052])
 def test_odd_ranks(oracle, K):
     d = synth.uniform_random(300, 500, 0.05, K=K, seed=40 + K)
-    for kernel in ("row", "lds"):
+    for kernel in ("row", "lds", "panel"):
         out, info = run_gpu(d, tile_x=64, kernel=KERNELS[kernel])
         check(d, out, oracle)
+        if kernel == "panel":
+            assert info["kernel"] == (capi.KERNEL_PANEL if K % 32 == 0 else capi.KERNEL_ROW_GATHER)
 
 
 def test_edge_shapes(oracle):
@@ -104,7 +108,7 @@ def test_edge_shapes(oracle):
                  val=torch.from_numpy(rng.standard_normal(len(r)).astype(np.float32)),
                  W=torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32)),
                  H=torch.from_numpy(rng.standard_normal((m, K)).astype(np.float32)))
-        for kernel, tx, ty in (("row", 0, 0), ("lds", 7, 3), ("lds", 300, 1)):
+        for kernel, tx, ty in (("row", 0, 0), ("lds", 7, 3), ("lds", 300, 1), ("panel", 7, 3), ("panel", 0, 0)):
             out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=KERNELS[kernel])
             check(d, out, oracle)
 
@@ -116,7 +120,7 @@ def test_empty_matrix_and_empty_rows(oracle):
     assert plan.info()["nnz"] == 0
     d = synth.uniform_random(2000, 100, 0.002, K=32, seed=9)  # most rows empty
     assert (np.diff(d["row_ptr"].numpy()) == 0).mean() > 0.5
-    for kernel in ("row", "lds"):
+    for kernel in ("row", "lds", "panel"):
         out, _ = run_gpu(d, tile_x=16, tile_y=5, kernel=KERNELS[kernel])
         check(d, out, oracle)
 
@@ -124,7 +128,7 @@ def test_empty_matrix_and_empty_rows(oracle):
 def test_closed_forms_on_gpu():
     d = synth.make(1)
     dev = torch.device("cuda:0")
-    for kernel in ("row", "lds"):
+    for kernel in ("row", "lds", "panel"):
         for K in (32, 100, 7):
             S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
             plan = S.plan(K, 256, 64, KERNELS[kernel])
@@ -151,7 +155,7 @@ def test_value_sources_and_host_form(oracle):
     check(d, out_a, oracle)
     # (b) a plan over a device-resident CSR, no values: out = dot (the shipping reference's form)
     rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
-    for kernel in (capi.KERNEL_ROW_GATHER, capi.KERNEL_LDS_TILE):
+    for kernel in (capi.KERNEL_ROW_GATHER, capi.KERNEL_LDS_TILE, capi.KERNEL_PANEL):
         plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, 128, 32,
                                          kernel, keep=(rp, ci))
         Wd = d["W"].to(dev); Hd = d["H"].to(dev); out = torch.empty(d["nnz"], device=dev)
@@ -189,6 +193,7 @@ def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
     out4, _ = run_gpu(d2, kernel=capi.KERNEL_ROW_GATHER)
     assert np.array_equal(out4, base * 4.0)
     _, absp = oracle.sddmm_f64(d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy(), d["W"].numpy(), d["H"].numpy())
-    for tx, ty in ((160, 50000), (50, 10), (1, 1), (12419, 1500)):
-        out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=capi.KERNEL_LDS_TILE)
-        assert parity_report(out, base, d["K"], absp)["violations"] == 0, (tx, ty)
+    for kernel in (capi.KERNEL_LDS_TILE, capi.KERNEL_PANEL):
+        for tx, ty in ((160, 50000), (50, 10), (1, 1), (12419, 1500)):
+            out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=kernel)
+            assert parity_report(out, base, d["K"], absp)["violations"] == 0, (kernel, tx, ty)
