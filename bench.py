@@ -82,7 +82,7 @@ def main():
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--K", type=int, default=None)
-    ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds", "panel"])
+    ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds", "panel", "hybrid"])
     ap.add_argument("--tile-x", type=int, default=0)
     ap.add_argument("--tile-y", type=int, default=0)
     ap.add_argument("--sweep-k", action="store_true", help="also report K = 32, 128, 256, 512")
@@ -99,7 +99,7 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}[args.kernel]
+    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL, "hybrid": capi.KERNEL_HYBRID}[args.kernel]
     names = {1: "uniform 4096^2 1%", 2: "bag-of-words 1500x12419", 3: "recommender 480189x17770 ~100M nnz",
              4: "R-MAT 2^22 ~200M nnz", 5: "banded 2^20 64/row"}
 
@@ -151,10 +151,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": names[args.config] + (f" (scale {args.scale})" if args.scale != 1.0 else ""),
                    "n_rows": d["n_rows"], "n_cols": d["n_cols"], "nnz": d["nnz"], "K": K0, "seed": d["seed"],
-                   "kernel": {1: "row_gather", 2: "lds_tile", 3: "panel"}[info["kernel"]],
+                   "kernel": {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid"}[info["kernel"]],
                    "tile_size_x": info["tile_size_x"], "tile_size_y": info["tile_size_y"],
                    "lanes_per_nnz": info["lanes_per_nnz"], "grid": info["grid"], "block": info["block"],
-                   "lds_bytes": info["lds_bytes"], "plan_ms": round(info["plan_ms"], 1)},
+                   "lds_bytes": info["lds_bytes"], "n_launches": info["n_launches"],
+                   "class_nnz_lds_panel_row": info["class_nnz"], "class_rows_lds_panel_row": info["class_rows"],
+                   "plan_ms": round(info["plan_ms"], 1)},
         "roofline": {"bound": "hbm", "achieved": round(main_res["alg_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(main_res["frac"], 4), "traffic": None,
                      "alg_bytes_per_launch": main_res["alg_bytes"], "kernel_ms": round(main_res["kernel_ms_mean"], 5)},

@@ -37,12 +37,14 @@ enum {
 };
 
 /* Kernel families a plan can be pinned to (sddmm_plan_create flags, low byte).
- * AUTO lets the planner choose from the matrix shape, K and the tile sizes. */
+ * AUTO lets the planner choose from the matrix shape, K and the tile sizes
+ * (it builds a HYBRID plan, which may consist of a single family). */
 enum {
     SDDMM_KERNEL_AUTO = 0,
     SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM */
     SDDMM_KERNEL_LDS_TILE = 2,   /* column tiles of H staged in LDS, W row (re)loaded per row run */
-    SDDMM_KERNEL_PANEL = 3       /* row panels of W resident in VGPRs, column tiles of H swept through LDS */
+    SDDMM_KERNEL_PANEL = 3,      /* row panels of W resident in VGPRs, column tiles of H swept through LDS */
+    SDDMM_KERNEL_HYBRID = 4      /* rows split by length: long -> LDS_TILE, medium -> PANEL, short -> ROW_GATHER */
 };
 
 typedef struct sddmm_coo sddmm_coo;   /* host-side sparse matrix (COO, int32/int32/fp32) */
@@ -56,12 +58,16 @@ typedef struct sddmm_plan_info {
     int32_t tile_size_y;  /* row-panel height actually used */
     int32_t k_slice;      /* K elements of each H row resident in LDS at a time (== K: no slicing) */
     int32_t n_col_tiles, n_row_panels;
-    int32_t kernel;       /* SDDMM_KERNEL_* actually chosen */
+    int32_t kernel;       /* SDDMM_KERNEL_* actually chosen (HYBRID: more than one launch) */
+    int32_t n_launches;   /* kernel launches per sddmm_execute */
     int32_t lanes_per_nnz;
     int32_t lds_bytes;    /* LDS per workgroup of the main kernel */
     int32_t grid, block;  /* launch shape of the main kernel */
     int64_t n_blocks;     /* (row panel, column tile) work items with at least one nonzero */
     int64_t device_bytes; /* device memory owned by the plan */
+    int64_t class_nnz[3]; /* nonzeros handled by LDS_TILE, PANEL, ROW_GATHER launches */
+    int64_t class_rows[3];
+    int64_t padded_positions; /* stream positions of the LDS_TILE launches, padding included */
     double plan_ms;       /* host time spent in the tiling pass + upload */
 } sddmm_plan_info;
 

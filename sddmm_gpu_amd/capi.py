@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsddmm_hip.so")
 
 OK, ERR_ARG, ERR_IO, ERR_FORMAT, ERR_RANGE, ERR_UNSORTED, ERR_HIP, ERR_NOMEM = range(8)
-KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL, KERNEL_HYBRID = 0, 1, 2, 3, 4
 
 
 class SddmmError(RuntimeError):
@@ -28,12 +28,13 @@ class SddmmError(RuntimeError):
 class PlanInfo(C.Structure):
     _fields_ = [("n_rows", c_int64), ("n_cols", c_int64), ("nnz", c_int64), ("rows_touched", c_int64),
                 ("cols_touched", c_int64), ("K", c_int32), ("tile_size_x", c_int32), ("tile_size_y", c_int32),
-                ("k_slice", c_int32), ("n_col_tiles", c_int32), ("n_row_panels", c_int32), ("kernel", c_int32),
+                ("k_slice", c_int32), ("n_col_tiles", c_int32), ("n_row_panels", c_int32), ("kernel", c_int32), ("n_launches", c_int32),
                 ("lanes_per_nnz", c_int32), ("lds_bytes", c_int32), ("grid", c_int32), ("block", c_int32),
-                ("n_blocks", c_int64), ("device_bytes", c_int64), ("plan_ms", c_double)]
+                ("n_blocks", c_int64), ("device_bytes", c_int64), ("class_nnz", c_int64 * 3), ("class_rows", c_int64 * 3), ("padded_positions", c_int64),
+                ("plan_ms", c_double)]
 
     def as_dict(self):
-        return {f: getattr(self, f) for f, _ in self._fields_}
+        return {f: (list(getattr(self, f)) if f.startswith("class_") else getattr(self, f)) for f, _ in self._fields_}
 
 
 class TilingView(C.Structure):

@@ -31,36 +31,32 @@ int upload(T **dst, const std::vector<T> &src, int64_t *bytes)
 
 }  // namespace
 
+// One kernel launch of a plan.  A plan is a list of launches over disjoint
+// sets of rows; together they write every nonzero's output exactly once.
+struct Launch {
+    int kind = 0;            // SDDMM_KERNEL_ROW_GATHER / LDS_TILE / PANEL
+    KernelFn fn = nullptr;   // stream kernels
+    PanelFn pfn = nullptr;   // panel kernel
+    TileFn tfn = nullptr;    // tile kernel (values in stream order)
+    TileFn tfn_val = nullptr, tfn_noval = nullptr;  // same, values in sorted order / no values
+    KArgs ka{};
+    PanelArgs pa{};
+    TileArgs ta{};
+    const float *sval = nullptr;  // the plan's values in stream order (LDS_TILE)
+    int32_t grid = 0, block = 0, lds = 0, k_slice = 0;
+    int64_t nnz = 0, rows = 0;
+};
+
 struct sddmm_plan {
     sddmm_plan_info info{};
-    Variant variant{0, 0, false};
-    KernelFn fn = nullptr;
-    const int32_t *d_col = nullptr;
-    bool own_col = false;
+    std::vector<Launch> launches;
+    std::vector<void *> owned;  // device allocations freed with the plan
+    const int32_t *d_row_ptr = nullptr, *d_col = nullptr;
     float *d_val = nullptr;
-    int32_t *d_perm = nullptr, *d_seg_row = nullptr, *d_batch_seg = nullptr;
-    uint64_t *d_batch_mask = nullptr;
-    WorkItem *d_items = nullptr;
-    int32_t n_items = 0;
-    int32_t chunk = 0;
-    // panel kernel
-    PanelFn panel_fn = nullptr;
-    const int32_t *d_row_ptr = nullptr;
-    bool own_row_ptr = false;
-    int32_t *d_slot_row = nullptr, *d_panel_tiles = nullptr;
-    int32_t n_panels = 0;
+    int32_t requested_kernel = 0;
     ~sddmm_plan()
     {
-        if (own_row_ptr && d_row_ptr) (void)hipFree((void *)d_row_ptr);
-        if (d_slot_row) (void)hipFree(d_slot_row);
-        if (d_panel_tiles) (void)hipFree(d_panel_tiles);
-        if (own_col && d_col) (void)hipFree((void *)d_col);
-        if (d_val) (void)hipFree(d_val);
-        if (d_perm) (void)hipFree(d_perm);
-        if (d_seg_row) (void)hipFree(d_seg_row);
-        if (d_batch_seg) (void)hipFree(d_batch_seg);
-        if (d_batch_mask) (void)hipFree(d_batch_mask);
-        if (d_items) (void)hipFree(d_items);
+        for (void *p : owned) (void)hipFree(p);
     }
 };
 
@@ -79,24 +75,31 @@ void build_batches(const std::vector<WorkItem> &items, const int32_t *seg_end, i
     }
     batch_seg.assign((size_t)nb_total, 0);
     batch_mask.assign((size_t)nb_total, 0);
+    auto fill = [&](const WorkItem &wi, int64_t b_lo, int64_t b_hi) {
+        int64_t s = std::upper_bound(seg_end, seg_end + n_seg, (int32_t)(wi.begin + b_lo * 64)) - seg_end;
+        for (int64_t b = b_lo; b < b_hi; ++b) {
+            int64_t p0 = wi.begin + b * 64, p1 = std::min<int64_t>(p0 + 64, wi.end);
+            while (s < n_seg && seg_end[s] <= p0) ++s;
+            batch_seg[wi.batch_base + b] = (int32_t)s;
+            uint64_t m = 0;
+            int64_t t = s;
+            while (t < n_seg && seg_end[t] < p1) {  // segment t+1 starts at seg_end[t], inside (p0, p1)
+                if (seg_end[t] > p0) m |= 1ull << (seg_end[t] - p0);
+                ++t;
+            }
+            batch_mask[wi.batch_base + b] = m;
+        }
+    };
+    if (items.size() == 1) {  // one long item: split its batches over the threads
+        const WorkItem &wi = items[0];
+        int64_t nb = ((int64_t)wi.end - wi.begin + 63) / 64;
+        parallel_ranges(nb, 1 << 12, [&](int64_t lo, int64_t hi, int) { fill(wi, lo, hi); });
+        return;
+    }
     parallel_ranges((int64_t)items.size(), 4, [&](int64_t ib, int64_t ie, int) {
         for (int64_t k = ib; k < ie; ++k) {
             const WorkItem &wi = items[k];
-            if (wi.end <= wi.begin) continue;
-            int64_t s = std::upper_bound(seg_end, seg_end + n_seg, wi.begin) - seg_end;  // segment of wi.begin
-            int64_t nb = ((int64_t)wi.end - wi.begin + 63) / 64;
-            for (int64_t b = 0; b < nb; ++b) {
-                int64_t p0 = wi.begin + b * 64, p1 = std::min<int64_t>(p0 + 64, wi.end);
-                while (s < n_seg && seg_end[s] <= p0) ++s;
-                batch_seg[wi.batch_base + b] = (int32_t)s;
-                uint64_t m = 0;
-                int64_t t = s;
-                while (t < n_seg && seg_end[t] < p1) {  // segment t+1 starts at seg_end[t], inside (p0, p1)
-                    if (seg_end[t] > p0) m |= 1ull << (seg_end[t] - p0);
-                    ++t;
-                }
-                batch_mask[wi.batch_base + b] = m;
-            }
+            if (wi.end > wi.begin) fill(wi, 0, ((int64_t)wi.end - wi.begin + 63) / 64);
         }
     });
 }
@@ -126,11 +129,356 @@ int device_ok()
     return SDDMM_OK;
 }
 
-// Common plan builder from host CSR arrays.  d_col_borrowed != null: the
-// device already holds col_ind.
+// Everything the launch builders need.
+struct Ctx {
+    sddmm_plan *P;
+    int64_t n_rows, n_cols, nnz;
+    const int32_t *row_ptr, *col_ind;  // host CSR
+    const float *vals;                 // host values or null
+    int32_t K;
+    int cus;
+    int64_t dev_bytes = 0;
+
+    template <class T>
+    int up(T **dst, const std::vector<T> &src)
+    {
+        int rc = upload(dst, src, &dev_bytes);
+        if (rc == SDDMM_OK && *dst) P->owned.push_back((void *)*dst);
+        return rc;
+    }
+    int need_row_ptr()
+    {
+        if (P->d_row_ptr) return SDDMM_OK;
+        int32_t *d = nullptr;
+        HIP_TRY(hipMalloc((void **)&d, (size_t)(n_rows + 1) * 4));
+        P->owned.push_back(d);
+        HIP_TRY(hipMemcpy(d, row_ptr, (size_t)(n_rows + 1) * 4, hipMemcpyHostToDevice));
+        dev_bytes += (n_rows + 1) * 4;
+        P->d_row_ptr = d;
+        return SDDMM_OK;
+    }
+};
+
+int64_t list_nnz(const Ctx &c, const std::vector<int32_t> &rows)
+{
+    int64_t n = 0;
+    for (int32_t r : rows) n += c.row_ptr[r + 1] - c.row_ptr[r];
+    return n;
+}
+
+// Row-gather launch over the given non-empty rows (ascending).  all_rows: the
+// list is every non-empty row of S, so the stream is S itself.
+int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
+{
+    Launch L;
+    L.kind = SDDMM_KERNEL_ROW_GATHER;
+    L.rows = (int64_t)rows.size();
+    const int64_t n = all_rows ? c.nnz : list_nnz(c, rows);
+    L.nnz = n;
+    if (n == 0) return SDDMM_OK;
+    const bool vec4 = c.K % 4 == 0;
+    Variant var = vec4 ? pick_variant(c.K, false) : Variant{0, 0, false};
+    L.fn = var.G ? stream_kernel(var, false) : generic_kernel();
+    if (!L.fn) return fail(SDDMM_ERR_ARG, "plan: no row-gather kernel for K = %d", c.K);
+    std::vector<int32_t> seg_end(rows.size()), perm;
+    int64_t acc = 0;
+    for (size_t i = 0; i < rows.size(); ++i) {
+        acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
+        seg_end[i] = (int32_t)acc;
+    }
+    if (!all_rows) {
+        perm.resize((size_t)n);
+        parallel_ranges((int64_t)rows.size(), 1 << 10, [&](int64_t b, int64_t e, int) {
+            for (int64_t i = b; i < e; ++i) {
+                int64_t d = i ? seg_end[i - 1] : 0;
+                for (int32_t p = c.row_ptr[rows[i]]; p < c.row_ptr[rows[i] + 1]; ++p) perm[d++] = p;
+            }
+        });
+    }
+    std::vector<int32_t> batch_seg;
+    std::vector<uint64_t> batch_mask;
+    std::vector<WorkItem> one{{0, (int32_t)n, 0, -1}};  // batches are multiples of 64 from 0
+    build_batches(one, seg_end.data(), (int64_t)seg_end.size(), batch_seg, batch_mask);
+    KArgs &a = L.ka;
+    int32_t *d_seg_row = nullptr, *d_perm = nullptr, *d_bseg = nullptr;
+    uint64_t *d_bmask = nullptr;
+    if (!(all_rows && (int64_t)rows.size() == c.n_rows))
+        if (int rc = c.up(&d_seg_row, rows)) return rc;
+    if (int rc = c.up(&d_perm, perm)) return rc;
+    if (int rc = c.up(&d_bseg, batch_seg)) return rc;
+    if (int rc = c.up(&d_bmask, batch_mask)) return rc;
+    a.seg_row = d_seg_row; a.perm = d_perm; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
+    a.nnz = (int32_t)n;
+    a.chunk = 64 * kRowGatherBatchesPerWave * (kRowGatherBlock / 64);
+    a.K = c.K; a.n_cols = (int32_t)c.n_cols; a.tile_x = (int32_t)c.n_cols;
+    a.generic_perm = var.G == 0;
+    L.grid = (int32_t)((n + a.chunk - 1) / a.chunk);
+    L.block = kRowGatherBlock;
+    L.k_slice = c.K;
+    c.P->info.lanes_per_nnz = var.G ? var.G : 8;
+    c.P->launches.push_back(L);
+    return SDDMM_OK;
+}
+
+// LDS-tile launch: the rows' nonzeros in tile order (tiles of x columns).
+int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x, int32_t y, sddmm_plan_info *I)
+{
+    Launch L;
+    L.kind = SDDMM_KERNEL_LDS_TILE;
+    L.rows = (int64_t)rows.size();
+    Variant var = pick_variant(c.K, true);
+    L.fn = var.G ? stream_kernel(var, true) : nullptr;
+    if (!L.fn) return fail(SDDMM_ERR_ARG, "plan: no LDS-tile kernel for K = %d", c.K);
+    sddmm_tiling T;
+    if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, y, T, all_rows ? nullptr : rows.data(),
+                              (int64_t)rows.size()))
+        return rc;
+    const int64_t n = T.nnz;
+    L.nnz = n;
+    if (n == 0) return SDDMM_OK;
+    // work items: row panels, cut further so that no item exceeds max_item nonzeros
+    const int64_t max_item = std::max<int64_t>(64 * 16 * 4, 8 * (int64_t)x);
+    std::vector<WorkItem> items;
+    int64_t nbatch = 0, n_blocks = 0;
+    for (int32_t j = 0; j < T.n_tiles; ++j) {
+        int64_t begin = T.tile_ptr[j];
+        for (int64_t b = T.block_ptr[j]; b < T.block_ptr[j + 1]; ++b) {
+            int64_t end = T.block_end[b];
+            ++n_blocks;
+            int64_t parts = std::max<int64_t>(1, (end - begin + max_item - 1) / max_item);
+            int64_t per = (((end - begin + parts - 1) / parts) + 63) / 64 * 64;
+            for (int64_t s = begin; s < end; s += per) {
+                int64_t e = std::min(end, s + per);
+                items.push_back({(int32_t)s, (int32_t)e, (int32_t)nbatch, j});
+                nbatch += (e - s + 63) / 64;
+            }
+            begin = end;
+        }
+    }
+    std::vector<int32_t> batch_seg;
+    std::vector<uint64_t> batch_mask;
+    build_batches(items, T.active_end.data(), (int64_t)T.active_end.size(), batch_seg, batch_mask);
+    // column indices (and the plan's own values) once more in tile order: coalesced reads
+    std::vector<int32_t> scol((size_t)n);
+    parallel_ranges(n, 1 << 16, [&](int64_t b, int64_t e, int) {
+        for (int64_t i = b; i < e; ++i) scol[i] = c.col_ind[T.tiled_ind[i]];
+    });
+    std::vector<float> sval;
+    if (c.vals) {
+        sval.resize((size_t)n);
+        parallel_ranges(n, 1 << 16, [&](int64_t b, int64_t e, int) {
+            for (int64_t i = b; i < e; ++i) sval[i] = c.vals[T.tiled_ind[i]];
+        });
+    }
+    KArgs &a = L.ka;
+    int32_t *d_perm = nullptr, *d_seg_row = nullptr, *d_bseg = nullptr, *d_scol = nullptr;
+    uint64_t *d_bmask = nullptr;
+    WorkItem *d_items = nullptr;
+    float *d_sval = nullptr;
+    if (int rc = c.up(&d_perm, T.tiled_ind)) return rc;
+    if (int rc = c.up(&d_seg_row, T.active_row)) return rc;
+    if (int rc = c.up(&d_items, items)) return rc;
+    if (int rc = c.up(&d_bseg, batch_seg)) return rc;
+    if (int rc = c.up(&d_bmask, batch_mask)) return rc;
+    if (int rc = c.up(&d_scol, scol)) return rc;
+    if (int rc = c.up(&d_sval, sval)) return rc;
+    a.perm = d_perm; a.seg_row = d_seg_row; a.items = d_items; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
+    a.scol = d_scol;
+    L.sval = d_sval;
+    a.n_items = (int32_t)items.size();
+    a.nnz = (int32_t)n; a.K = c.K; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
+    L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)items.size()));
+    L.block = kLdsBlock;
+    L.lds = (int32_t)((int64_t)x * c.K * 4);
+    L.k_slice = c.K;
+    HIP_TRY(hipFuncSetAttribute((const void *)L.fn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (I) {
+        I->tile_size_x = x; I->tile_size_y = y; I->n_col_tiles = T.n_tiles;
+        I->n_row_panels = (int32_t)((T.max_active_rows + y - 1) / y);
+        I->n_blocks = n_blocks; I->lanes_per_nnz = var.G; I->lds_bytes = L.lds; I->grid = L.grid; I->block = L.block;
+    }
+    c.P->launches.push_back(L);
+    return SDDMM_OK;
+}
+
+// Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
+// (row, tile) run padded to a multiple of G stream positions.
+int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x, int want_g, sddmm_plan_info *I)
+{
+    Launch L;
+    L.kind = SDDMM_KERNEL_LDS_TILE;
+    L.rows = (int64_t)rows.size();
+    const TileVariant tv = pick_tile_variant(c.K, want_g);
+    L.tfn = tv.G ? tile_kernel(tv, 0) : nullptr;
+    if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
+    L.tfn_val = tile_kernel(tv, 1);
+    L.tfn_noval = tile_kernel(tv, 2);
+    const int G = tv.G;
+    sddmm_tiling T;
+    if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, INT32_MAX, T,
+                              all_rows ? nullptr : rows.data(), (int64_t)rows.size()))
+        return rc;
+    L.nnz = T.nnz;
+    if (T.nnz == 0) return SDDMM_OK;
+    const int64_t n_seg = (int64_t)T.active_end.size();
+    std::vector<int64_t> poff((size_t)n_seg + 1);
+    std::vector<int32_t> seg_tile((size_t)n_seg);
+    poff[0] = 0;
+    for (int32_t j = 0; j < T.n_tiles; ++j)
+        for (int64_t s = T.active_ptr[j]; s < T.active_ptr[j + 1]; ++s) {
+            const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
+            const int64_t len = T.active_end[s] - b;
+            poff[s + 1] = poff[s] + (len + G - 1) / G * G;
+            seg_tile[s] = j;
+        }
+    const int64_t np = poff[n_seg];
+    if (np >= INT32_MAX - 4096) return fail(SDDMM_ERR_RANGE, "plan: padded stream beyond int32 offsets");
+    std::vector<int32_t> perm((size_t)np), scol((size_t)np), grow((size_t)(np / G));
+    std::vector<float> sval;
+    if (c.vals) sval.resize((size_t)np);
+    parallel_ranges(n_seg, 1 << 10, [&](int64_t sb, int64_t se, int) {
+        for (int64_t s = sb; s < se; ++s) {
+            const int32_t j = seg_tile[s];
+            const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
+            const int64_t len = T.active_end[s] - b;
+            const int32_t pad_col = (int32_t)((int64_t)j * x);
+            int64_t d = poff[s];
+            for (int64_t i = 0; i < len; ++i, ++d) {
+                const int32_t p = T.tiled_ind[b + i];
+                perm[d] = p;
+                scol[d] = c.col_ind[p];
+                if (c.vals) sval[d] = c.vals[p];
+            }
+            for (; d < poff[s + 1]; ++d) {
+                perm[d] = -1;
+                scol[d] = pad_col;
+                if (c.vals) sval[d] = 0.f;
+            }
+            for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
+        }
+    });
+    // first padded stream position of each tile
+    std::vector<int32_t> tptr((size_t)T.n_tiles + 1);
+    int64_t n_blocks = 0;
+    for (int32_t j = 0; j <= T.n_tiles; ++j) tptr[j] = (int32_t)poff[T.active_ptr[j]];
+    for (int32_t j = 0; j < T.n_tiles; ++j) n_blocks += tptr[j + 1] > tptr[j];
+    TileArgs &a = L.ta;
+    int32_t *d_perm = nullptr, *d_scol = nullptr, *d_grow = nullptr;
+    float *d_sval = nullptr;
+    int32_t *d_tptr = nullptr;
+    if (int rc = c.up(&d_perm, perm)) return rc;
+    if (int rc = c.up(&d_scol, scol)) return rc;
+    if (int rc = c.up(&d_grow, grow)) return rc;
+    if (int rc = c.up(&d_sval, sval)) return rc;
+    if (int rc = c.up(&d_tptr, tptr)) return rc;
+    a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.tile_ptr = d_tptr;
+    L.sval = d_sval;
+    a.n_tiles = T.n_tiles; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
+    L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
+    L.block = kLdsBlock;
+    L.lds = (int32_t)((int64_t)x * c.K * 4);
+    L.k_slice = c.K;
+    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_val, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_noval, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (I) {
+        I->tile_size_x = x; I->tile_size_y = (int32_t)std::min<int64_t>(c.n_rows, INT32_MAX); I->n_col_tiles = T.n_tiles;
+        I->n_row_panels = 1; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
+        I->grid = L.grid; I->block = L.block;
+    }
+    c.P->info.padded_positions += np;
+    c.P->launches.push_back(L);
+    return SDDMM_OK;
+}
+
+// Panel launch over the given non-empty rows (ascending): K slices of ks.
+int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, int32_t tile_y, sddmm_plan_info *I)
+{
+    Launch L;
+    L.kind = SDDMM_KERNEL_PANEL;
+    L.rows = (int64_t)rows.size();
+    L.nnz = list_nnz(c, rows);
+    if (L.nnz == 0) return SDDMM_OK;
+    const PanelVariant pv = pick_panel_variant(ks);
+    L.pfn = panel_kernel(pv);
+    if (!L.pfn) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", ks);
+    const int32_t fit = kLdsMaxBytes / (ks * 4);
+    int32_t x = tile_x > 0 ? std::min(tile_x, fit) : fit;
+    x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(c.n_cols, 1));
+    const int octs_cap = pv.S * pv.NWAVES;  // octets (8 rows, one per lane group of a wave) per panel
+    int octs = octs_cap;
+    if (tile_y > 0) octs = (int)std::max<int64_t>(1, std::min<int64_t>(octs_cap, ((int64_t)tile_y + 7) / 8));
+    // spread a small row set over the CUs rather than filling few panels to the brim
+    {
+        int64_t want_panels = std::min<int64_t>(c.cus, ((int64_t)rows.size() + 63) / 64);
+        int64_t octs_even = (((int64_t)rows.size() + want_panels - 1) / want_panels + 7) / 8;
+        if (tile_y <= 0) octs = (int)std::max<int64_t>(1, std::min<int64_t>(octs, octs_even));
+    }
+    const int rows_per_panel = octs * 8;
+    // panels: contiguous runs of the rows (keeps the column locality of neighbouring
+    // rows); inside a panel rows are ranked by length so that the 8 groups of a
+    // wave work on rows of similar length in the same slot
+    const int64_t n_panels = ((int64_t)rows.size() + rows_per_panel - 1) / rows_per_panel;
+    std::vector<int32_t> slot_row((size_t)n_panels * pv.S * pv.NWAVES * 8, -1);
+    std::vector<int32_t> panel_tiles((size_t)n_panels * 2, 0);
+    const int32_t *row_ptr = c.row_ptr, *col_ind = c.col_ind;
+    parallel_ranges(n_panels, 4, [&](int64_t pb, int64_t pe, int) {
+        std::vector<int32_t> rk;
+        for (int64_t p = pb; p < pe; ++p) {
+            const int64_t b = p * rows_per_panel, e = std::min<int64_t>(b + rows_per_panel, (int64_t)rows.size());
+            rk.assign(rows.begin() + b, rows.begin() + e);
+            std::stable_sort(rk.begin(), rk.end(), [&](int32_t u, int32_t v) {
+                return row_ptr[u + 1] - row_ptr[u] > row_ptr[v + 1] - row_ptr[v];
+            });
+            int32_t cmin = INT32_MAX, cmax = 0;
+            for (size_t i = 0; i < rk.size(); ++i) {
+                const int oct = (int)(i / 8), g = (int)(i % 8);
+                const int slot = oct / pv.NWAVES, wave = oct % pv.NWAVES;
+                slot_row[((((size_t)p * pv.S + slot) * pv.NWAVES) + wave) * 8 + g] = rk[i];
+                cmin = std::min(cmin, col_ind[row_ptr[rk[i]]]);
+                cmax = std::max(cmax, col_ind[row_ptr[rk[i] + 1] - 1]);
+            }
+            panel_tiles[2 * p] = cmin / x;
+            panel_tiles[2 * p + 1] = cmax / x;
+        }
+    });
+    if (int rc = c.need_row_ptr()) return rc;
+    int32_t *d_slot = nullptr, *d_pt = nullptr;
+    if (int rc = c.up(&d_slot, slot_row)) return rc;
+    if (int rc = c.up(&d_pt, panel_tiles)) return rc;
+    PanelArgs &pa = L.pa;
+    pa.slot_row = d_slot; pa.panel_tiles = d_pt;
+    pa.n_panels = (int32_t)n_panels; pa.tile_x = x; pa.n_cols = (int32_t)c.n_cols; pa.K = c.K;
+    L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>(c.cus, n_panels));
+    L.block = pv.NWAVES * 64;
+    L.lds = x * ks * 4;
+    L.k_slice = ks;
+    HIP_TRY(hipFuncSetAttribute((const void *)L.pfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (I) {
+        I->tile_size_x = x; I->tile_size_y = rows_per_panel; I->k_slice = ks;
+        I->n_col_tiles = (int32_t)((c.n_cols + x - 1) / x); I->n_row_panels = (int32_t)n_panels;
+        I->n_blocks = 0;
+        for (int64_t p = 0; p < n_panels; ++p) I->n_blocks += panel_tiles[2 * p + 1] - panel_tiles[2 * p] + 1;
+        I->lanes_per_nnz = 8; I->grid = L.grid; I->block = L.block; I->lds_bytes = L.lds;
+    }
+    c.P->launches.push_back(L);
+    return SDDMM_OK;
+}
+
+int64_t env_i64(const char *name, int64_t dflt)
+{
+    const char *e = getenv(name);
+    if (!e || !*e) return dflt;
+    char *end = nullptr;
+    long long v = strtoll(e, &end, 10);
+    return (end && *end == 0) ? (int64_t)v : dflt;
+}
+
+// Common plan builder from host CSR arrays.  d_*_borrowed != null: the device
+// already holds that array.
 int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr, const int32_t *col_ind,
-              const float *vals, const int32_t *d_row_ptr_borrowed, const int32_t *d_col_borrowed, int32_t K, int32_t tile_x, int32_t tile_y,
-              uint32_t flags, sddmm_plan **out)
+              const float *vals, const int32_t *d_row_ptr_borrowed, const int32_t *d_col_borrowed, int32_t K,
+              int32_t tile_x, int32_t tile_y, uint32_t flags, sddmm_plan **out)
 {
     auto t0 = std::chrono::steady_clock::now();
     if (K < 1) return fail(SDDMM_ERR_ARG, "plan: K must be >= 1 (got %d)", K);
@@ -141,7 +489,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         return fail(SDDMM_ERR_RANGE, "plan: dense factor too large");
     if (int rc = device_ok()) return rc;
     int want = (int)(flags & 0xff);
-    if (want > SDDMM_KERNEL_PANEL) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
+    if (want > SDDMM_KERNEL_HYBRID) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
 
     sddmm_plan *P = new (std::nothrow) sddmm_plan;
     if (!P) return fail(SDDMM_ERR_NOMEM, "plan: out of memory");
@@ -149,179 +497,138 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     sddmm_plan_info &I = P->info;
     I.n_rows = n_rows; I.n_cols = n_cols; I.nnz = nnz; I.K = K; I.k_slice = K;
     count_touched(n_rows, n_cols, nnz, row_ptr, col_ind, &I.rows_touched, &I.cols_touched);
+    P->requested_kernel = want;
 
-    const bool vec4 = (K % 4 == 0);
-    Variant var = vec4 ? pick_variant(K) : Variant{0, 0, false};
-    const bool have_fast = var.G != 0;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, 0));
+    Ctx c{P, n_rows, n_cols, nnz, row_ptr, col_ind, vals, K, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
 
-    // kernel choice
-    int kernel = want;
-    const int64_t row_bytes = (int64_t)K * 4;
-    int32_t fit_x = (int32_t)std::min<int64_t>(kLdsMaxBytes / row_bytes, INT32_MAX);
-    if (kernel == SDDMM_KERNEL_AUTO)
-        kernel = (have_fast && tile_x > 0 && tile_x < n_cols && fit_x >= 8) ? SDDMM_KERNEL_LDS_TILE : SDDMM_KERNEL_ROW_GATHER;
-    if (kernel == SDDMM_KERNEL_LDS_TILE && (!have_fast || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
-    // the panel kernel works on K slices of 128, 64 or 32 elements
-    const int ks = (K % 128 == 0) ? 128 : (K % 64 == 0) ? 64 : (K % 32 == 0) ? 32 : 0;
-    if (kernel == SDDMM_KERNEL_PANEL && ks == 0) kernel = SDDMM_KERNEL_ROW_GATHER;
-    I.kernel = kernel;
-    I.lanes_per_nnz = have_fast ? var.G : 8;
-    P->variant = var;
-
-    int64_t dev_bytes = 0;
+    P->d_row_ptr = d_row_ptr_borrowed;
     if (d_col_borrowed) {
         P->d_col = d_col_borrowed;
-    } else {
+    } else if (nnz) {
         int32_t *d = nullptr;
-        if (nnz) {
-            HIP_TRY(hipMalloc((void **)&d, (size_t)nnz * 4));
-            HIP_TRY(hipMemcpy(d, col_ind, (size_t)nnz * 4, hipMemcpyHostToDevice));
-            dev_bytes += nnz * 4;
-        }
-        P->d_col = d; P->own_col = true;
+        HIP_TRY(hipMalloc((void **)&d, (size_t)nnz * 4));
+        P->owned.push_back(d);
+        HIP_TRY(hipMemcpy(d, col_ind, (size_t)nnz * 4, hipMemcpyHostToDevice));
+        c.dev_bytes += nnz * 4;
+        P->d_col = d;
     }
     if (vals && nnz) {
         HIP_TRY(hipMalloc((void **)&P->d_val, (size_t)nnz * 4));
+        P->owned.push_back(P->d_val);
         HIP_TRY(hipMemcpy(P->d_val, vals, (size_t)nnz * 4, hipMemcpyHostToDevice));
-        dev_bytes += nnz * 4;
+        c.dev_bytes += nnz * 4;
     }
 
-    std::vector<int32_t> batch_seg;
-    std::vector<uint64_t> batch_mask;
-    if (kernel == SDDMM_KERNEL_PANEL) {
-        const PanelVariant pv = pick_panel_variant(ks);
-        P->panel_fn = panel_kernel(pv);
-        if (!P->panel_fn) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", ks);
-        const int32_t fit = kLdsMaxBytes / (ks * 4);
-        int32_t x = tile_x > 0 ? std::min(tile_x, fit) : fit;
-        x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
-        const int octs_cap = pv.S * pv.NWAVES;  // octets (8 rows, one per lane group of a wave) per panel
-        int octs = octs_cap;
-        if (tile_y > 0) octs = (int)std::max<int64_t>(1, std::min<int64_t>(octs_cap, ((int64_t)tile_y + 7) / 8));
-        const int rows_per_panel = octs * 8;
-        // panels: contiguous runs of non-empty rows (keeps the column locality of
-        // neighbouring rows); inside a panel rows are ranked by length so that the
-        // 8 groups of a wave work on rows of similar length in the same slot
-        std::vector<int32_t> ne;
-        ne.reserve((size_t)I.rows_touched);
-        for (int64_t r = 0; r < n_rows; ++r)
-            if (row_ptr[r + 1] > row_ptr[r]) ne.push_back((int32_t)r);
-        const int64_t n_panels = ((int64_t)ne.size() + rows_per_panel - 1) / rows_per_panel;
-        std::vector<int32_t> slot_row((size_t)n_panels * pv.S * pv.NWAVES * 8, -1);
-        std::vector<int32_t> panel_tiles((size_t)n_panels * 2, 0);
-        parallel_ranges(n_panels, 4, [&](int64_t pb, int64_t pe, int) {
-            std::vector<int32_t> rk;
-            for (int64_t p = pb; p < pe; ++p) {
-                const int64_t b = p * rows_per_panel, e = std::min<int64_t>(b + rows_per_panel, (int64_t)ne.size());
-                rk.assign(ne.begin() + b, ne.begin() + e);
-                std::stable_sort(rk.begin(), rk.end(), [&](int32_t u, int32_t v) {
-                    return row_ptr[u + 1] - row_ptr[u] > row_ptr[v + 1] - row_ptr[v];
-                });
+    // non-empty rows, ascending
+    std::vector<int32_t> ne;
+    ne.reserve((size_t)I.rows_touched);
+    for (int64_t r = 0; r < n_rows; ++r)
+        if (row_ptr[r + 1] > row_ptr[r]) ne.push_back((int32_t)r);
+
+    const bool have_vec = (K % 4 == 0) && pick_variant(K, true).G != 0;
+    const int64_t row_bytes = (int64_t)K * 4;
+    const int32_t fit_x = (int32_t)std::min<int64_t>(kLdsMaxBytes / row_bytes, INT32_MAX);  // H rows per LDS tile at full K
+    const int ks = (K % 128 == 0) ? 128 : (K % 64 == 0) ? 64 : (K % 32 == 0) ? 32 : 0;    // panel kernel K slice
+
+    int kernel = want;
+    if (kernel == SDDMM_KERNEL_AUTO) kernel = SDDMM_KERNEL_HYBRID;
+    if (kernel == SDDMM_KERNEL_LDS_TILE && (!have_vec || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
+    if (kernel == SDDMM_KERNEL_PANEL && ks == 0) kernel = SDDMM_KERNEL_ROW_GATHER;
+
+    I.tile_size_x = (int32_t)std::min<int64_t>(n_cols, INT32_MAX);
+    I.tile_size_y = (int32_t)std::min<int64_t>(n_rows, INT32_MAX);
+    I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1; I.lanes_per_nnz = 8;
+
+    if (kernel == SDDMM_KERNEL_HYBRID) {
+        // Rows are split by length into up to three classes, each with the
+        // kernel whose on-chip reuse pays for it:
+        //   long   (>= long_min nonzeros):  LDS-tile stream; each (row, tile) run is long
+        //          enough to amortise re-reading the W row once per tile
+        //   medium : panel kernel; the W row stays in VGPRs across all tiles
+        //   short  (< short_max nonzeros):  row gather; too few nonzeros per tile for a
+        //          staged H tile to be reused
+        // Column span of a row panel (not n_cols) decides how many tiles a panel sweeps.
+        const PanelVariant pv = ks ? pick_panel_variant(ks) : PanelVariant{0, 0, 0};
+        const int64_t panel_rows = ks ? (int64_t)pv.S * pv.NWAVES * 8 : 1;
+        double span = (double)n_cols;
+        if (!ne.empty()) {  // mean column span of panels of consecutive rows
+            double acc = 0; int64_t cnt = 0;
+            for (size_t b = 0; b < ne.size(); b += (size_t)panel_rows * 16) {  // every 16th panel
+                size_t e = std::min(ne.size(), b + (size_t)panel_rows);
                 int32_t cmin = INT32_MAX, cmax = 0;
-                for (size_t i = 0; i < rk.size(); ++i) {
-                    const int oct = (int)(i / 8), g = (int)(i % 8);
-                    const int slot = oct / pv.NWAVES, wave = oct % pv.NWAVES;
-                    slot_row[((((size_t)p * pv.S + slot) * pv.NWAVES) + wave) * 8 + g] = rk[i];
-                    cmin = std::min(cmin, col_ind[row_ptr[rk[i]]]);
-                    cmax = std::max(cmax, col_ind[row_ptr[rk[i] + 1] - 1]);
+                for (size_t i = b; i < e; ++i) {
+                    cmin = std::min(cmin, col_ind[row_ptr[ne[i]]]);
+                    cmax = std::max(cmax, col_ind[row_ptr[ne[i] + 1] - 1]);
                 }
-                panel_tiles[2 * p] = cmin / x;
-                panel_tiles[2 * p + 1] = cmax / x;
+                acc += (double)(cmax - cmin + 1); ++cnt;
             }
-        });
-        if (d_row_ptr_borrowed) {
-            P->d_row_ptr = d_row_ptr_borrowed;
-        } else {
-            int32_t *d = nullptr;
-            HIP_TRY(hipMalloc((void **)&d, (size_t)(n_rows + 1) * 4));
-            HIP_TRY(hipMemcpy(d, row_ptr, (size_t)(n_rows + 1) * 4, hipMemcpyHostToDevice));
-            dev_bytes += (n_rows + 1) * 4;
-            P->d_row_ptr = d; P->own_row_ptr = true;
+            span = acc / (double)cnt;
         }
-        if (int rc = upload(&P->d_slot_row, slot_row, &dev_bytes)) return rc;
-        if (int rc = upload(&P->d_panel_tiles, panel_tiles, &dev_bytes)) return rc;
-        P->n_panels = (int32_t)n_panels;
-        hipDeviceProp_t prop;
-        HIP_TRY(hipGetDeviceProperties(&prop, 0));
-        const int cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        I.tile_size_x = x; I.tile_size_y = rows_per_panel; I.k_slice = ks;
-        I.n_col_tiles = (int32_t)((n_cols + x - 1) / x); I.n_row_panels = (int32_t)n_panels;
-        I.n_blocks = 0;
-        for (int64_t p = 0; p < n_panels; ++p) I.n_blocks += panel_tiles[2 * p + 1] - panel_tiles[2 * p] + 1;
-        I.lanes_per_nnz = 8;
-        I.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>(cus, n_panels));
-        I.block = pv.NWAVES * 64;
-        I.lds_bytes = x * ks * 4;
-        HIP_TRY(hipFuncSetAttribute((const void *)P->panel_fn, hipFuncAttributeMaxDynamicSharedMemorySize, I.lds_bytes));
-        I.device_bytes = dev_bytes;
-        I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-        guard.p = nullptr;
-        *out = P;
-        return SDDMM_OK;
-    }
-    if (kernel == SDDMM_KERNEL_ROW_GATHER) {
-        // segments = non-empty rows
-        std::vector<int32_t> seg_end, seg_row;
-        seg_end.reserve((size_t)I.rows_touched); seg_row.reserve((size_t)I.rows_touched);
-        for (int64_t r = 0; r < n_rows; ++r)
-            if (row_ptr[r + 1] > row_ptr[r]) { seg_end.push_back(row_ptr[r + 1]); seg_row.push_back((int32_t)r); }
-        P->chunk = 64 * kRowGatherBatchesPerWave * (kRowGatherBlock / 64);
-        std::vector<WorkItem> one{{0, (int32_t)nnz, 0, -1}};  // batches are global multiples of 64
-        build_batches(one, seg_end.data(), (int64_t)seg_end.size(), batch_seg, batch_mask);
-        if (I.rows_touched != n_rows)
-            if (int rc = upload(&P->d_seg_row, seg_row, &dev_bytes)) return rc;
-        I.tile_size_x = (int32_t)std::min<int64_t>(n_cols, INT32_MAX); I.tile_size_y = (int32_t)std::min<int64_t>(n_rows, INT32_MAX);
-        I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1;
-        I.grid = (int32_t)((nnz + P->chunk - 1) / P->chunk);
-        I.block = kRowGatherBlock; I.lds_bytes = 0;
-        P->fn = have_fast ? stream_kernel(var, false) : generic_kernel();
-    } else {
-        int32_t x = tile_x > 0 ? tile_x : fit_x;
-        x = std::min(x, fit_x);
+        int32_t xa = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
+        const double tiles_a = std::max(1.0, span / std::max(1, xa));
+        int64_t long_min = (have_vec && fit_x >= 8) ? (int64_t)(16.0 * tiles_a) : INT64_MAX;
+        int64_t short_max = (have_vec && fit_x >= 8) ? (int64_t)std::max(8.0, 2.0 * tiles_a) : INT64_MAX;
+        (void)panel_rows;
+        long_min = env_i64("SDDMM_LONG_ROW_MIN", long_min);
+        short_max = env_i64("SDDMM_SHORT_ROW_MAX", short_max);
+        if (short_max > long_min) short_max = long_min;
+        std::vector<int32_t> rl, rm, rs;
+        int64_t nl = 0, nm = 0, nsh = 0;
+        for (int32_t r : ne) {
+            const int64_t d = row_ptr[r + 1] - row_ptr[r];
+            if (d >= long_min) { rl.push_back(r); nl += d; }
+            else if (d >= short_max) { rm.push_back(r); nm += d; }
+            else { rs.push_back(r); nsh += d; }
+        }
+        // classes too small to fill the machine join a neighbour
+        if (!rm.empty() && (nm * 50 < nnz || (int64_t)rm.size() < 64)) {
+            rs.insert(rs.end(), rm.begin(), rm.end()); nsh += nm; rm.clear(); nm = 0;
+            std::sort(rs.begin(), rs.end());
+        }
+        if (!rl.empty() && nl * 50 < nnz) {
+            auto &dst = rm.empty() ? rs : rm;
+            dst.insert(dst.end(), rl.begin(), rl.end());
+            (rm.empty() ? nsh : nm) += nl; rl.clear(); nl = 0;
+            std::sort(dst.begin(), dst.end());
+        }
+        sddmm_plan_info scratch{};
+        const bool tile_ok = pick_tile_variant(K, 0).G != 0;
+        if (!rl.empty()) {
+            if (tile_ok) { if (int rc = add_tile(c, rl, rl.size() == ne.size(), xa, (int)env_i64("SDDMM_TILE_G", 0), &I)) return rc; }
+            else if (int rc = add_lds_tile(c, rl, rl.size() == ne.size(), xa, tile_y > 0 ? tile_y : (int32_t)std::min<int64_t>(n_rows, INT32_MAX), &I)) return rc;
+        }
+        if (!rm.empty()) {
+            const bool med_tile = tile_ok && fit_x >= 8 && pick_tile_variant(K, 4).G != 0 && env_i64("SDDMM_MEDIUM_PANEL", 0) == 0;
+            if (med_tile) { if (int rc = add_tile(c, rm, rm.size() == ne.size(), xa, 4, rl.empty() ? &I : &scratch)) return rc; }
+            else if (int rc = add_panel(c, rm, ks, tile_x, tile_y, rl.empty() ? &I : &scratch)) return rc;
+        }
+        if (!rs.empty())
+            if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
+        I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
+        I.class_nnz[0] = nl; I.class_nnz[1] = nm; I.class_nnz[2] = nsh;
+        I.class_rows[0] = (int64_t)rl.size(); I.class_rows[1] = (int64_t)rm.size(); I.class_rows[2] = (int64_t)rs.size();
+    } else if (kernel == SDDMM_KERNEL_PANEL) {
+        if (int rc = add_panel(c, ne, ks, tile_x, tile_y, &I)) return rc;
+        I.kernel = kernel; I.class_nnz[1] = nnz; I.class_rows[1] = (int64_t)ne.size();
+    } else if (kernel == SDDMM_KERNEL_LDS_TILE) {
+        int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
         x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
         int32_t y = tile_y > 0 ? tile_y : (int32_t)std::min<int64_t>(std::max<int64_t>(n_rows, 1), INT32_MAX);
-        sddmm_tiling T;
-        if (int rc = build_tiling(n_rows, n_cols, nnz, row_ptr, col_ind, x, y, T)) return rc;
-        // work items: row panels, cut further so that no item exceeds max_item nonzeros
-        const int64_t max_item = std::max<int64_t>(64 * 16 * 4, 8 * (int64_t)x);
-        std::vector<WorkItem> items;
-        int64_t nbatch = 0, n_blocks = 0;
-        for (int32_t j = 0; j < T.n_tiles; ++j) {
-            int64_t begin = T.tile_ptr[j];
-            for (int64_t b = T.block_ptr[j]; b < T.block_ptr[j + 1]; ++b) {
-                int64_t end = T.block_end[b];
-                ++n_blocks;
-                int64_t parts = std::max<int64_t>(1, (end - begin + max_item - 1) / max_item);
-                int64_t per = (((end - begin + parts - 1) / parts) + 63) / 64 * 64;
-                for (int64_t s = begin; s < end; s += per) {
-                    int64_t e = std::min(end, s + per);
-                    items.push_back({(int32_t)s, (int32_t)e, (int32_t)nbatch, j});
-                    nbatch += (e - s + 63) / 64;
-                }
-                begin = end;
-            }
-        }
-        build_batches(items, T.active_end.data(), (int64_t)T.active_end.size(), batch_seg, batch_mask);
-        if (int rc = upload(&P->d_perm, T.tiled_ind, &dev_bytes)) return rc;
-        if (int rc = upload(&P->d_seg_row, T.active_row, &dev_bytes)) return rc;
-        if (int rc = upload(&P->d_items, items, &dev_bytes)) return rc;
-        P->n_items = (int32_t)items.size();
-        I.tile_size_x = x; I.tile_size_y = y; I.n_col_tiles = T.n_tiles;
-        I.n_row_panels = (int32_t)((T.max_active_rows + y - 1) / y);
-        I.n_blocks = n_blocks;
-        hipDeviceProp_t prop;
-        HIP_TRY(hipGetDeviceProperties(&prop, 0));
-        int cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-        I.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)cus, (int64_t)items.size()));
-        I.block = kLdsBlock;
-        I.lds_bytes = (int32_t)((int64_t)x * row_bytes);
-        P->fn = stream_kernel(var, true);
-        HIP_TRY(hipFuncSetAttribute((const void *)P->fn, hipFuncAttributeMaxDynamicSharedMemorySize, I.lds_bytes));
+        if (pick_tile_variant(K, 0).G != 0 && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
+            if (int rc = add_tile(c, ne, true, x, 0, &I)) return rc;
+            I.tile_size_y = y;
+        } else if (int rc = add_lds_tile(c, ne, true, x, y, &I)) return rc;
+        I.kernel = kernel; I.class_nnz[0] = nnz; I.class_rows[0] = (int64_t)ne.size();
+    } else {
+        if (int rc = add_row_gather(c, ne, true)) return rc;
+        I.kernel = SDDMM_KERNEL_ROW_GATHER; I.class_nnz[2] = nnz; I.class_rows[2] = (int64_t)ne.size();
     }
-    if (!P->fn) return fail(SDDMM_ERR_ARG, "plan: no kernel for K = %d", K);
-    if (int rc = upload(&P->d_batch_seg, batch_seg, &dev_bytes)) return rc;
-    if (int rc = upload(&P->d_batch_mask, batch_mask, &dev_bytes)) return rc;
-    I.device_bytes = dev_bytes;
+    if (!P->launches.empty() && I.grid == 0) { I.grid = P->launches[0].grid; I.block = P->launches[0].block; I.lds_bytes = P->launches[0].lds; }
+    I.n_launches = 0;
+    for (const Launch &L : P->launches) I.n_launches += (L.kind == SDDMM_KERNEL_PANEL) ? K / L.k_slice : 1;
+    I.device_bytes = c.dev_bytes;
     I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     guard.p = nullptr;
     *out = P;
@@ -404,42 +711,38 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
     const sddmm_plan_info &I = plan->info;
     if (I.nnz == 0) return SDDMM_OK;
     if (!d_W || !d_H || !d_out) return fail(SDDMM_ERR_ARG, "sddmm_execute: NULL device pointer");
-    if (((uintptr_t)d_W | (uintptr_t)d_H) & 15u)
-        if (I.K % 4 == 0 && (plan->variant.G || I.kernel == SDDMM_KERNEL_PANEL))
-            return fail(SDDMM_ERR_ARG, "sddmm_execute: W and H must be 16-byte aligned");
-    if (I.kernel == SDDMM_KERNEL_PANEL) {
-        PanelArgs pa{};
-        pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
-        pa.val = d_val ? d_val : plan->d_val;
-        pa.W = d_W; pa.H = d_H; pa.out = d_out;
-        pa.slot_row = plan->d_slot_row; pa.panel_tiles = plan->d_panel_tiles;
-        pa.n_panels = plan->n_panels; pa.tile_x = I.tile_size_x; pa.n_cols = (int32_t)I.n_cols; pa.K = I.K;
-        for (int k_off = 0; k_off < I.K; k_off += I.k_slice) {
-            pa.k_off = k_off;
-            pa.accumulate = k_off > 0;
-            hipLaunchKernelGGL(plan->panel_fn, dim3((unsigned)I.grid), dim3((unsigned)I.block), (size_t)I.lds_bytes,
-                               (hipStream_t)stream, pa);
+    if ((((uintptr_t)d_W | (uintptr_t)d_H) & 15u) && I.K % 4 == 0)
+        return fail(SDDMM_ERR_ARG, "sddmm_execute: W and H must be 16-byte aligned");
+    const float *val = d_val ? d_val : plan->d_val;
+    for (const Launch &L : plan->launches) {
+        if (L.kind == SDDMM_KERNEL_PANEL) {
+            PanelArgs pa = L.pa;
+            pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
+            pa.val = val; pa.W = d_W; pa.H = d_H; pa.out = d_out;
+            for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
+                pa.k_off = k_off;
+                pa.accumulate = k_off > 0;
+                hipLaunchKernelGGL(L.pfn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
+                                   (hipStream_t)stream, pa);
+            }
+        } else if (L.tfn) {
+            TileArgs ta = L.ta;
+            ta.val = val;
+            ta.sval = d_val ? nullptr : L.sval;
+            ta.W = d_W; ta.H = d_H; ta.out = d_out;
+            const TileFn fn = ta.sval ? L.tfn : (val ? L.tfn_val : L.tfn_noval);
+            hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
+                               (hipStream_t)stream, ta);
+        } else {
+            KArgs a = L.ka;
+            a.col_ind = plan->d_col;
+            a.val = val;
+            a.sval = d_val ? nullptr : L.sval;
+            a.W = d_W; a.H = d_H; a.out = d_out;
+            hipLaunchKernelGGL(L.fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
+                               (hipStream_t)stream, a);
         }
-        HIP_TRY(hipGetLastError());
-        return SDDMM_OK;
     }
-    KArgs a{};
-    a.col_ind = plan->d_col;
-    a.val = d_val ? d_val : plan->d_val;
-    a.W = d_W; a.H = d_H; a.out = d_out;
-    a.perm = plan->d_perm;
-    a.seg_row = plan->d_seg_row;
-    a.batch_seg = plan->d_batch_seg;
-    a.batch_mask = plan->d_batch_mask;
-    a.items = plan->d_items;
-    a.n_items = plan->n_items;
-    a.nnz = (int32_t)I.nnz;
-    a.chunk = plan->chunk;
-    a.K = I.K;
-    a.tile_x = I.tile_size_x;
-    a.n_cols = (int32_t)I.n_cols;
-    hipLaunchKernelGGL(plan->fn, dim3((unsigned)I.grid), dim3((unsigned)I.block), (size_t)I.lds_bytes,
-                       (hipStream_t)stream, a);
     HIP_TRY(hipGetLastError());
     return SDDMM_OK;
 }

@@ -49,6 +49,7 @@ void build_row_ptr(const sddmm_coo &S, std::vector<int32_t> &row_ptr);
 
 // The tiling pass proper, on raw CSR arrays (host).
 int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
-                 const int32_t *col_ind, int32_t tile_x, int32_t tile_y, sddmm_tiling &T);
+                 const int32_t *col_ind, int32_t tile_x, int32_t tile_y, sddmm_tiling &T,
+                 const int32_t *row_list, int64_t n_list);
 
 }  // namespace sddmm

@@ -17,6 +17,8 @@ struct KArgs {
     const float *W, *H;
     float *out;
     const int32_t *perm;       // stream position -> sorted position, null = identity
+    const int32_t *scol;       // column indices in stream order, or null (use col_ind[perm])
+    const float *sval;         // values in stream order, or null (use val[perm])
     const int32_t *seg_row;    // segment -> global row, null = identity
     const int32_t *batch_seg;  // per batch: segment of its first nonzero
     const uint64_t *batch_mask;  // per batch: bit L (L >= 1) set if lane L starts a new segment
@@ -27,6 +29,7 @@ struct KArgs {
     int32_t K;
     int32_t tile_x;
     int32_t n_cols;
+    int32_t generic_perm;
 };
 
 constexpr int kRowGatherBlock = 256;   // 4 waves
@@ -39,6 +42,28 @@ struct Variant {
     bool exact;   // K == 4*G*KPL
 };
 using KernelFn = void (*)(const KArgs);
+
+// Tile kernel: padded tile-order stream, H tiles in LDS.
+struct TileArgs {
+    const int32_t *perm;   // stream position -> sorted position, -1 = padding
+    const int32_t *scol;   // column of each stream position (padding: first column of the tile)
+    const int32_t *grow;   // row of each group of G consecutive stream positions
+    const float *sval;     // values in stream order (padding: 0) or null
+    const float *val;      // values in sorted order or null
+    const float *W, *H;
+    float *out;
+    const int32_t *tile_ptr;  // [n_tiles+1] first stream position of each column tile
+    int32_t n_tiles;
+    int32_t tile_x, n_cols;
+};
+struct TileVariant {
+    int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL
+};
+using TileFn = void (*)(const TileArgs);
+// want_g > 0: that group size or nothing; 0: the preferred one for K
+TileVariant pick_tile_variant(int K, int want_g);
+// vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
+TileFn tile_kernel(const TileVariant &v, int vmode);
 
 // Panel kernel: rows of W resident in VGPRs, column tiles of H in LDS.
 struct PanelArgs {
@@ -62,7 +87,7 @@ PanelVariant pick_panel_variant(int k_slice);
 PanelFn panel_kernel(const PanelVariant &v);
 
 // lanes per nonzero and float4 slots per lane for a given K (K % 4 == 0); G == 0: none
-Variant pick_variant(int K);
+Variant pick_variant(int K, bool lds_tile);
 KernelFn stream_kernel(const Variant &v, bool lds_tile);
 KernelFn generic_kernel();
 

@@ -17,6 +17,7 @@
 // together by a butterfly of cross-lane exchanges that leaves nonzero i's dot
 // product in lane i, which scales it by S.val and stores it.
 #include <hip/hip_runtime.h>
+#include <utility>
 #include "kernels.hpp"
 
 using namespace sddmm;
@@ -32,29 +33,64 @@ __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float ac
     return acc;
 }
 
+// value held by lane I of the caller's group of G lanes
+template <int G, int I>
+__device__ __forceinline__ int group_bcast(int v)
+{
+    if constexpr (G <= 32)
+        return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // src = (lane & ~(G-1)) | I
+    else
+        return __shfl(v, I, G);
+}
+
+// value of lane (lane ^ S)
+template <int S>
+__device__ __forceinline__ float xor_lane(float v)
+{
+    if constexpr (S == 1)
+        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+    else if constexpr (S == 2)
+        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+    else if constexpr (S < 32)
+        return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (S << 10) | 0x1f));
+    else
+        return __shfl_xor(v, S, 64);
+}
+
 // Reduces G accumulators across the G lanes of a group so that lane i of the
 // group ends with the full sum of accumulator i (returned).
+template <int G, int S = G / 2>
+__device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
+{
+    if constexpr (S >= 1) {
+        const bool upper = (l & S) != 0;
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            float keep = upper ? acc[j + S] : acc[j];
+            float send = upper ? acc[j] : acc[j + S];
+            acc[j] = keep + xor_lane<S>(send);
+        }
+        transpose_reduce_step<G, S / 2>(acc, l);
+    }
+}
 template <int G>
 __device__ __forceinline__ float transpose_reduce(float (&acc)[G], int l)
 {
-#pragma unroll
-    for (int s = G / 2; s >= 1; s >>= 1) {
-        const bool upper = (l & s) != 0;
-#pragma unroll
-        for (int j = 0; j < s; ++j) {
-            float keep = upper ? acc[j + s] : acc[j];
-            float send = upper ? acc[j] : acc[j + s];
-            acc[j] = keep + __shfl_xor(send, s, G);
-        }
-    }
+    transpose_reduce_step<G>(acc, l);
     return acc[0];
 }
+
+struct Batch {
+    int row, p, col;  // row < 0: lane holds no nonzero
+    float v;
+};
 
 // K = 4 * (number of float4 per row); each lane of a group owns KPL float4
 // slots of a row: slot j sits at float4 index (((j + rot) % KPL) * G + l).  `rot`
 // differs between the groups that share one 16-lane LDS access phase, so that
 // their 16-byte reads fall into different banks when rows are a multiple of
 // 256 bytes apart.  EXACT: K == 4*G*KPL (no slot is out of range).
+// The index data of batch b+1 is requested before batch b is computed.
 template <int G, int KPL, bool EXACT, bool LDS_TILE>
 __global__ __launch_bounds__(LDS_TILE ? kLdsBlock : kRowGatherBlock)
 void sddmm_stream_kernel(const KArgs a)
@@ -69,6 +105,7 @@ void sddmm_stream_kernel(const KArgs a)
     const int l = lane & (G - 1);
     const int rot = (lane / G) & ROT_MASK;
     const int K4 = a.K >> 2;
+    const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
 
     int slot[KPL];
 #pragma unroll
@@ -111,33 +148,35 @@ void sddmm_stream_kernel(const KArgs a)
         const int nb = (end - begin + 63) >> 6;
         const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
 
+        auto load_batch = [&](int bi) -> Batch {
+            Batch b{-1, 0, 0, 0.f};
+            const int pos = begin + (bi << 6) + lane;
+            if (bi < b1 && pos < end) {
+                const int gb = batch_base + bi;
+                const int seg = a.batch_seg[gb] + __popcll(a.batch_mask[gb] & le);
+                b.row = a.seg_row ? a.seg_row[seg] : seg;
+                b.p = a.perm ? a.perm[pos] : pos;
+                b.col = a.scol ? a.scol[pos] : a.col_ind[b.p];
+                b.v = a.sval ? a.sval[pos] : (a.val ? a.val[b.p] : 1.0f);
+            }
+            return b;
+        };
+
         int cur_row = -1;
         float4 w[KPL];
 #pragma unroll
         for (int j = 0; j < KPL; ++j) w[j] = make_float4(0.f, 0.f, 0.f, 0.f);
 
+        Batch nxt = load_batch(b0);
         for (int bi = b0; bi < b1; ++bi) {
-            const int pos = begin + (bi << 6) + lane;
-            const bool valid = pos < end;
-            const int gb = batch_base + bi;
-            const int seg0 = a.batch_seg[gb];
-            const uint64_t mask = a.batch_mask[gb];
-            const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
-            const int seg = seg0 + __popcll(mask & le);
-            int row = -1, p = 0, col = 0;
-            float v = 0.f;
-            if (valid) {
-                row = a.seg_row ? a.seg_row[seg] : seg;
-                p = a.perm ? a.perm[pos] : pos;
-                col = a.col_ind[p];
-                v = a.val ? a.val[p] : 1.0f;
-            }
+            const Batch cur = nxt;
+            nxt = load_batch(bi + 1);
             float acc[G];
 #pragma unroll
             for (int i = 0; i < G; ++i) acc[i] = 0.f;
 
-            const int row_first = __shfl(row, 0, G);
-            const int row_last = __shfl(row, G - 1, G);
+            const int row_first = group_bcast<G, 0>(cur.row);
+            const int row_last = group_bcast<G, G - 1>(cur.row);
             if (row_first == row_last && row_last >= 0) {
                 // all G nonzeros of this group lie in one row: no checks inside
                 if (row_first != cur_row) {
@@ -147,38 +186,40 @@ void sddmm_stream_kernel(const KArgs a)
                     for (int j = 0; j < KPL; ++j)
                         w[j] = (EXACT || slot[j] < K4) ? wr[slot[j]] : make_float4(0.f, 0.f, 0.f, 0.f);
                 }
-#pragma unroll
-                for (int i = 0; i < G; ++i) {
-                    const int c_i = __shfl(col, i, G);
-                    const float4 *hr = LDS_TILE ? (lds_tile + (size_t)(c_i - tile_base) * K4)
-                                                : (H4 + (size_t)c_i * K4);
-#pragma unroll
-                    for (int j = 0; j < KPL; ++j)
-                        if (EXACT || slot[j] < K4) acc[i] = dot4(w[j], hr[slot[j]], acc[i]);
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < G; ++i) {
-                    const int r_i = __shfl(row, i, G);
-                    const int c_i = __shfl(col, i, G);
-                    if (r_i >= 0) {
-                        if (r_i != cur_row) {
-                            cur_row = r_i;
-                            const float4 *wr = W4 + (size_t)cur_row * K4;
-#pragma unroll
-                            for (int j = 0; j < KPL; ++j)
-                                w[j] = (EXACT || slot[j] < K4) ? wr[slot[j]] : make_float4(0.f, 0.f, 0.f, 0.f);
-                        }
+                [&]<int... I>(std::integer_sequence<int, I...>) {
+                    ((void)[&] {
+                        const int c_i = group_bcast<G, I>(cur.col);
                         const float4 *hr = LDS_TILE ? (lds_tile + (size_t)(c_i - tile_base) * K4)
                                                     : (H4 + (size_t)c_i * K4);
 #pragma unroll
                         for (int j = 0; j < KPL; ++j)
-                            if (EXACT || slot[j] < K4) acc[i] = dot4(w[j], hr[slot[j]], acc[i]);
-                    }
-                }
+                            if (EXACT || slot[j] < K4) acc[I] = dot4(w[j], hr[slot[j]], acc[I]);
+                    }(), ...);
+                }(std::make_integer_sequence<int, G>{});
+            } else {
+                [&]<int... I>(std::integer_sequence<int, I...>) {
+                    ((void)[&] {
+                        const int r_i = group_bcast<G, I>(cur.row);
+                        const int c_i = group_bcast<G, I>(cur.col);
+                        if (r_i >= 0) {
+                            if (r_i != cur_row) {
+                                cur_row = r_i;
+                                const float4 *wr = W4 + (size_t)cur_row * K4;
+#pragma unroll
+                                for (int j = 0; j < KPL; ++j)
+                                    w[j] = (EXACT || slot[j] < K4) ? wr[slot[j]] : make_float4(0.f, 0.f, 0.f, 0.f);
+                            }
+                            const float4 *hr = LDS_TILE ? (lds_tile + (size_t)(c_i - tile_base) * K4)
+                                                        : (H4 + (size_t)c_i * K4);
+#pragma unroll
+                            for (int j = 0; j < KPL; ++j)
+                                if (EXACT || slot[j] < K4) acc[I] = dot4(w[j], hr[slot[j]], acc[I]);
+                        }
+                    }(), ...);
+                }(std::make_integer_sequence<int, G>{});
             }
             const float sum = transpose_reduce<G>(acc, l);
-            if (valid) a.out[p] = sum * v;
+            if (cur.row >= 0) a.out[cur.p] = sum * cur.v;
         }
     }
 }
@@ -205,12 +246,13 @@ void sddmm_generic_kernel(const KArgs a)
         const uint64_t mask = a.batch_mask[gb];
         const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
         const int seg = a.batch_seg[gb] + __popcll(mask & le);
-        int row = -1, col = 0;
+        int row = -1, col = 0, p = 0;
         float v = 0.f;
         if (valid) {
             row = a.seg_row ? a.seg_row[seg] : seg;
-            col = a.col_ind[pos];
-            v = a.val ? a.val[pos] : 1.0f;
+            p = a.perm ? a.perm[pos] : pos;
+            col = a.col_ind[p];
+            v = a.val ? a.val[p] : 1.0f;
         }
         float acc[G];
 #pragma unroll
@@ -226,7 +268,7 @@ void sddmm_generic_kernel(const KArgs a)
             acc[i] = s;
         }
         const float sum = transpose_reduce<G>(acc, l);
-        if (valid) a.out[pos] = sum * v;
+        if (valid) a.out[p] = sum * v;
     }
 }
 
@@ -234,9 +276,16 @@ void sddmm_generic_kernel(const KArgs a)
 
 namespace sddmm {
 
-Variant pick_variant(int K)
+// With H in LDS fewer lanes per nonzero pay (less cross-lane work per FMA);
+// gathers from global memory prefer at least 8 lanes (128 contiguous bytes).
+Variant pick_variant(int K, bool lds_tile)
 {
     const int K4 = K / 4;
+    if (lds_tile) {
+        const int c4[][2] = {{4, 2}, {4, 4}, {4, 8}};
+        for (auto &c : c4)
+            if (c[0] * c[1] == K4) return {c[0], c[1], true};
+    }
     const int cand[][2] = {{8, 1}, {8, 2}, {8, 3}, {8, 4}, {8, 6}, {8, 8}, {16, 6}, {16, 8}, {32, 6}, {32, 8}, {64, 6}, {64, 8}};
     for (auto &c : cand)
         if (c[0] * c[1] == K4) return {c[0], c[1], true};
@@ -252,6 +301,7 @@ static KernelFn lookup(const Variant &v)
     if (v.G == g && v.KPL == kpl)                                                       \
         return v.exact ? (KernelFn)sddmm_stream_kernel<g, kpl, true, LDS_TILE>          \
                        : (KernelFn)sddmm_stream_kernel<g, kpl, false, LDS_TILE>;
+    SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8)
     SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 3) SDDMM_CASE(8, 4) SDDMM_CASE(8, 6) SDDMM_CASE(8, 8)
     SDDMM_CASE(16, 6) SDDMM_CASE(16, 8) SDDMM_CASE(32, 6) SDDMM_CASE(32, 8) SDDMM_CASE(64, 6) SDDMM_CASE(64, 8)
 #undef SDDMM_CASE

@@ -1,0 +1,211 @@
+// Tile kernel of the SDDMM engine for gfx950 (MI355X): column tiles of H in
+// LDS, nonzeros streamed in tile order with every (row, tile) run padded to a
+// multiple of G positions.
+//
+// The stream lists S tile by tile (tiles of tile_x columns), rows ascending
+// inside a tile.  Each run of one row inside one tile is padded with empty
+// positions to a multiple of G, so a group of G lanes always works on ONE row:
+// there is no per-nonzero row test in the inner loop.  A batch is 64
+// consecutive stream positions (one per lane).  While batch b is computed the
+// index data of batch b+1 (original position, column, value, row) and -- if
+// the group's row changes -- its W row slice are already in flight.  For each
+// of its G nonzeros a group reads the H row from LDS in contiguous 16-byte
+// pieces (groups sharing one 16-lane LDS phase start at different pieces, so
+// their reads fall into different banks), multiplies with the W slice held in
+// VGPRs, and a butterfly over the G lanes leaves nonzero i's dot product in
+// lane i, which scales it by S.val and stores it at the nonzero's own
+// position in the output.
+#include <hip/hip_runtime.h>
+#include <utility>
+#include "kernels.hpp"
+
+using namespace sddmm;
+
+namespace {
+
+__device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float acc)
+{
+    acc = fmaf(a.x, b.x, acc);
+    acc = fmaf(a.y, b.y, acc);
+    acc = fmaf(a.z, b.z, acc);
+    acc = fmaf(a.w, b.w, acc);
+    return acc;
+}
+
+template <int G, int I>
+__device__ __forceinline__ int group_bcast(int v)
+{
+    return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // src = (lane & ~(G-1)) | I
+}
+
+template <int S>
+__device__ __forceinline__ float xor_lane(float v)
+{
+    if constexpr (S == 1)
+        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+    else if constexpr (S == 2)
+        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+    else
+        return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (S << 10) | 0x1f));
+}
+
+template <int G, int S = G / 2>
+__device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
+{
+    if constexpr (S >= 1) {
+        const bool upper = (l & S) != 0;
+#pragma unroll
+        for (int j = 0; j < S; ++j) {
+            float keep = upper ? acc[j + S] : acc[j];
+            float send = upper ? acc[j] : acc[j + S];
+            acc[j] = keep + xor_lane<S>(send);
+        }
+        transpose_reduce_step<G, S / 2>(acc, l);
+    }
+}
+
+// VMODE: where S.val comes from -- 0: a.sval (stream order), 1: a.val (sorted
+// order, read through the position), 2: nowhere (no scaling).
+//
+// The loop is software-pipelined by hand and free of branches around loads, so
+// that every wait is for exactly the data needed: while batch b is computed,
+// the index data of batch b+2 and the W row slice of batch b+1 are in flight.
+template <int G, int KPL, int VMODE>
+__global__ __launch_bounds__(kLdsBlock)
+void sddmm_tile_kernel(const TileArgs a)
+{
+    extern __shared__ float4 lds_tile[];
+    constexpr int NW = kLdsBlock / 64;
+    constexpr int K4 = G * KPL;
+    constexpr int PHASE_GROUPS = (16 / G) >= 1 ? (16 / G) : 1;
+    constexpr int ROT_MASK = (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL) - 1;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int l = lane & (G - 1);
+    const int rot = (lane / G) & ROT_MASK;
+
+    int slot[KPL];
+#pragma unroll
+    for (int j = 0; j < KPL; ++j) slot[j] = (((j + rot) % KPL) * G + l);
+
+    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W);
+    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H);
+
+    // This workgroup's share of the stream: an equal, 64-aligned range of
+    // positions, walked tile by tile (usually one or two tiles).
+    const int64_t total = a.tile_ptr[a.n_tiles];
+    const int lo = (int)(((total * blockIdx.x / gridDim.x) + 63) & ~(int64_t)63);
+    const int hi = (blockIdx.x + 1 == gridDim.x) ? (int)total
+                                                 : (int)(((total * (blockIdx.x + 1) / gridDim.x) + 63) & ~(int64_t)63);
+    int tile = 0;
+    {   // first tile whose end lies beyond lo
+        int a0 = 0, a1 = a.n_tiles;
+        while (a0 < a1) {
+            const int mid = (a0 + a1) >> 1;
+            if (a.tile_ptr[mid + 1] <= lo) a0 = mid + 1; else a1 = mid;
+        }
+        tile = a0;
+    }
+    bool first = true;
+    for (; tile < a.n_tiles && a.tile_ptr[tile] < hi; ++tile) {
+        const int begin = max(lo, a.tile_ptr[tile]), end = min(hi, a.tile_ptr[tile + 1]);
+        if (end <= begin) continue;
+        const int tile_base = tile * a.tile_x;
+        {
+            if (!first) __syncthreads();  // everyone is done with the previous tile
+            first = false;
+            const int rows = min(a.tile_x, a.n_cols - tile_base);
+            const float4 *src = H4 + (size_t)tile_base * K4;
+            const int n4 = rows * K4;
+            for (int i = threadIdx.x; i < n4; i += kLdsBlock) lds_tile[i] = src[i];
+            __syncthreads();
+        }
+        const int nb = (end - begin + 63) >> 6;
+        const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
+        if (b0 >= b1) continue;  // (no barrier below this point inside the tile)
+
+        // index data of one batch; positions past the item are clamped into it
+        // (their results are discarded), so no load sits behind a branch
+        struct Meta { int row, p, col; float sv; };
+        auto issue_meta = [&](int bi) -> Meta {
+            const int pc = min(begin + (bi << 6) + lane, end - 1);
+            Meta m;
+            m.row = a.grow[pc / G];
+            m.p = a.perm[pc];
+            m.col = a.scol[pc];
+            m.sv = (VMODE == 0) ? a.sval[pc] : 1.0f;
+            return m;
+        };
+        auto issue_w = [&](float4 (&w)[KPL], int row) {
+            const float4 *wr = W4 + (size_t)row * K4;
+#pragma unroll
+            for (int j = 0; j < KPL; ++j) w[j] = wr[slot[j]];
+        };
+        auto compute = [&](const float4 (&w)[KPL], const Meta &m, int bi) {
+            float v = m.sv;
+            if (VMODE == 1) v = a.val[max(m.p, 0)];
+            float acc[G];
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                ((void)[&] {
+                    const int c_i = group_bcast<G, I>(m.col);
+                    const float4 *hr = lds_tile + (c_i - tile_base) * K4;
+                    float s = 0.f;
+#pragma unroll
+                    for (int j = 0; j < KPL; ++j) s = dot4(w[j], hr[slot[j]], s);
+                    acc[I] = s;
+                }(), ...);
+            }(std::make_integer_sequence<int, G>{});
+            transpose_reduce_step<G>(acc, l);
+            const int pos = begin + (bi << 6) + lane;
+            if (pos < end && m.p >= 0) a.out[m.p] = acc[0] * v;
+        };
+
+        float4 wa[KPL], wb[KPL];
+        Meta m0 = issue_meta(b0);
+        Meta m1 = issue_meta(b0 + 1);
+        issue_w(wa, m0.row);
+        for (int bi = b0; bi < b1; bi += 2) {
+            Meta m2 = issue_meta(bi + 2);
+            issue_w(wb, m1.row);
+            compute(wa, m0, bi);
+            if (bi + 1 >= b1) break;
+            Meta m3 = issue_meta(bi + 3);
+            issue_w(wa, m2.row);
+            compute(wb, m1, bi + 1);
+            m0 = m2;
+            m1 = m3;
+        }
+    }
+}
+
+}  // namespace
+
+namespace sddmm {
+
+TileVariant pick_tile_variant(int K, int want_g)
+{
+    if (K % 4) return {0, 0};
+    const int K4 = K / 4;
+    const int cand[][2] = {{4, 2}, {4, 4}, {4, 8}, {8, 1}, {8, 2}, {8, 4}, {8, 8}, {16, 4}, {16, 8}, {32, 4}, {32, 8}};
+    TileVariant best{0, 0};
+    for (auto &c : cand) {
+        if (c[0] * c[1] != K4) continue;
+        if (want_g > 0 ? c[0] == want_g : (best.G == 0 || c[1] == 4)) best = {c[0], c[1]};
+    }
+    return best;
+}
+
+TileFn tile_kernel(const TileVariant &v, int vmode)
+{
+#define SDDMM_CASE(g, kpl)                                                         \
+    if (v.G == g && v.KPL == kpl)                                                  \
+        return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0>                   \
+             : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1> : (TileFn)sddmm_tile_kernel<g, kpl, 2>;
+    SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
+    SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
+#undef SDDMM_CASE
+    return nullptr;
+}
+
+}  // namespace sddmm

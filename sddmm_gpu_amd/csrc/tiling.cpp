@@ -11,9 +11,18 @@
 
 namespace sddmm {
 
-int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
-                 const int32_t *col_ind, int32_t tile_x, int32_t tile_y, sddmm_tiling &T)
+int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz_all, const int32_t *row_ptr,
+                 const int32_t *col_ind, int32_t tile_x, int32_t tile_y, sddmm_tiling &T,
+                 const int32_t *row_list, int64_t n_list)
 {
+    // row_list != null: only those rows (ascending) take part; offsets then count their nonzeros only
+    const int64_t n_it = row_list ? n_list : n_rows;
+    auto row_of = [&](int64_t i) -> int64_t { return row_list ? row_list[i] : i; };
+    int64_t nnz = nnz_all;
+    if (row_list) {
+        nnz = 0;
+        for (int64_t i = 0; i < n_list; ++i) nnz += row_ptr[row_list[i] + 1] - row_ptr[row_list[i]];
+    }
     if (tile_x < 1 || tile_y < 1) return fail(SDDMM_ERR_ARG, "tiling: tile sizes must be >= 1");
     const int64_t n_tiles = std::max<int64_t>(1, (n_cols + tile_x - 1) / tile_x);
     if (n_tiles >= INT32_MAX) return fail(SDDMM_ERR_RANGE, "tiling: too many column tiles");
@@ -23,11 +32,21 @@ int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row
     // Threads own contiguous row ranges balanced by nonzeros.
     int nt = (int)std::max<int64_t>(1, std::min<int64_t>(hw_threads(), nnz / (1 << 15) + 1));
     std::vector<int64_t> rb((size_t)nt + 1);
-    rb[0] = 0; rb[nt] = n_rows;
-    for (int t = 1; t < nt; ++t) {
-        int64_t target = nnz * t / nt;
-        rb[t] = std::lower_bound(row_ptr, row_ptr + n_rows + 1, (int32_t)target) - row_ptr;
-        rb[t] = std::min<int64_t>(std::max(rb[t], rb[t - 1]), n_rows);
+    rb[0] = 0; rb[nt] = n_it;
+    if (row_list) {
+        int64_t acc = 0;
+        int t = 1;
+        for (int64_t i = 0; i < n_list && t < nt; ++i) {
+            acc += row_ptr[row_list[i] + 1] - row_ptr[row_list[i]];
+            while (t < nt && acc >= nnz * t / nt) rb[t++] = i + 1;
+        }
+        for (; t < nt; ++t) rb[t] = n_list;
+    } else {
+        for (int t = 1; t < nt; ++t) {
+            int64_t target = nnz * t / nt;
+            rb[t] = std::lower_bound(row_ptr, row_ptr + n_rows + 1, (int32_t)target) - row_ptr;
+            rb[t] = std::min<int64_t>(std::max(rb[t], rb[t - 1]), n_rows);
+        }
     }
     // pass 1: per thread, nonzeros and (row, tile) runs per tile
     std::vector<std::vector<int64_t>> cnt_nnz(nt, std::vector<int64_t>((size_t)n_tiles, 0));
@@ -41,7 +60,8 @@ int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row
     run_threads([&](int t) {
         auto &cn = cnt_nnz[t];
         auto &cs = cnt_seg[t];
-        for (int64_t r = rb[t]; r < rb[t + 1]; ++r) {
+        for (int64_t ri = rb[t]; ri < rb[t + 1]; ++ri) {
+            const int64_t r = row_of(ri);
             int64_t i = row_ptr[r], e = row_ptr[r + 1];
             while (i < e) {
                 int64_t tile = col_ind[i] / tile_x;
@@ -81,7 +101,8 @@ int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row
     run_threads([&](int t) {
         auto &on = off_nnz[t];
         auto &os = off_seg[t];
-        for (int64_t r = rb[t]; r < rb[t + 1]; ++r) {
+        for (int64_t ri = rb[t]; ri < rb[t + 1]; ++ri) {
+            const int64_t r = row_of(ri);
             int64_t i = row_ptr[r], e = row_ptr[r + 1];
             while (i < e) {
                 int64_t tile = col_ind[i] / tile_x;
@@ -140,7 +161,7 @@ extern "C" int sddmm_tiling_create(const sddmm_coo *S, int32_t tile_size_x, int3
     try {
         std::vector<int32_t> rp;
         build_row_ptr(*S, rp);
-        rc = build_tiling(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), tile_size_x, tile_size_y, *T);
+        rc = build_tiling(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), tile_size_x, tile_size_y, *T, nullptr, 0);
     } catch (const std::bad_alloc &) {
         rc = fail(SDDMM_ERR_NOMEM, "sddmm_tiling_create: out of memory");
     }

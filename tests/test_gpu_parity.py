@@ -12,7 +12,8 @@ from sddmm_gpu_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
 
-KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}
+KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL,
+           "hybrid": capi.KERNEL_HYBRID, "auto": capi.KERNEL_AUTO}
 
 
 def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_vals=True):
@@ -64,14 +65,16 @@ def test_config2_bag_of_words(oracle, kernel, tx, ty):
     d = synth.make(2)
     out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=KERNELS.get(kernel, capi.KERNEL_AUTO))
     rep = check(d, out, oracle)
+    if kernel == "lds":
+        assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] == 64
     if kernel == "auto":
-        assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] == 160  # 192 rows of K=256 exceed 160 KB
+        assert sum(info["class_nnz"]) == d["nnz"] and sum(info["class_rows"]) == info["rows_touched"]
     print(info, rep)
 
 
 @pytest.mark.parametrize("cfg,scale,K", [(3, 0.02, 128), (3, 0.02, 32), (3, 0.01, 256), (3, 0.005, 512),
                                          (4, 2.0 ** -7, 64), (5, 2.0 ** -6, 512), (5, 2.0 ** -7, 1024)])
-@pytest.mark.parametrize("kernel", ["row", "lds", "panel"])
+@pytest.mark.parametrize("kernel", ["row", "lds", "panel", "auto"])
 def test_scaled_configs(oracle, cfg, scale, K, kernel):
     d = synth.make(cfg, scale, K=K)
     out, info = run_gpu(d, kernel=KERNELS[kernel])
@@ -197,3 +200,20 @@ def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
         for tx, ty in ((160, 50000), (50, 10), (1, 1), (12419, 1500)):
             out, info = run_gpu(d, tile_x=tx, tile_y=ty, kernel=kernel)
             assert parity_report(out, base, d["K"], absp)["violations"] == 0, (kernel, tx, ty)
+
+
+@pytest.mark.parametrize("long_min,short_max", [(200, 20), (100, 100), (10 ** 9, 30), (50, 0)])
+def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
+    """Forces the three row classes (LDS-tile / panel / row-gather) of a hybrid
+    plan through the length thresholds and checks the union of their outputs."""
+    monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(long_min))
+    monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
+    d = synth.make(3, 0.02, K=128)
+    deg = np.diff(d["row_ptr"].numpy())
+    out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID)
+    check(d, out, oracle)
+    assert sum(info["class_nnz"]) == d["nnz"]
+    assert sum(info["class_rows"]) == int((deg > 0).sum())
+    if long_min == 200 and short_max == 20:
+        assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 3
+        assert info["class_rows"][0] == int((deg >= 200).sum())
