@@ -159,6 +159,15 @@ struct Ctx {
     }
 };
 
+int64_t env_i64(const char *name, int64_t dflt)
+{
+    const char *e = getenv(name);
+    if (!e || !*e) return dflt;
+    char *end = nullptr;
+    long long v = strtoll(e, &end, 10);
+    return (end && *end == 0) ? (int64_t)v : dflt;
+}
+
 int64_t list_nnz(const Ctx &c, const std::vector<int32_t> &rows)
 {
     int64_t n = 0;
@@ -309,10 +318,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
     L.kind = SDDMM_KERNEL_LDS_TILE;
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(c.K, want_g);
-    L.tfn = tv.G ? tile_kernel(tv, 0) : nullptr;
+    const int nwaves = (int)env_i64("SDDMM_TILE_WAVES", 16);
+    L.tfn = tv.G ? tile_kernel(tv, 0, nwaves) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
-    L.tfn_val = tile_kernel(tv, 1);
-    L.tfn_noval = tile_kernel(tv, 2);
+    L.tfn_val = tile_kernel(tv, 1, nwaves);
+    L.tfn_noval = tile_kernel(tv, 2, nwaves);
     const int G = tv.G;
     sddmm_tiling T;
     if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, INT32_MAX, T,
@@ -341,17 +351,18 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
             const int32_t j = seg_tile[s];
             const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
             const int64_t len = T.active_end[s] - b;
-            const int32_t pad_col = (int32_t)((int64_t)j * x);
+            const int32_t tile_base = (int32_t)((int64_t)j * x);
+            const int32_t row_bytes = c.K * 4;
             int64_t d = poff[s];
             for (int64_t i = 0; i < len; ++i, ++d) {
                 const int32_t p = T.tiled_ind[b + i];
                 perm[d] = p;
-                scol[d] = c.col_ind[p];
+                scol[d] = (c.col_ind[p] - tile_base) * row_bytes;  // byte offset of the H row inside the LDS tile
                 if (c.vals) sval[d] = c.vals[p];
             }
             for (; d < poff[s + 1]; ++d) {
                 perm[d] = -1;
-                scol[d] = pad_col;
+                scol[d] = 0;
                 if (c.vals) sval[d] = 0.f;
             }
             for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
@@ -375,7 +386,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
     L.sval = d_sval;
     a.n_tiles = T.n_tiles; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
-    L.block = kLdsBlock;
+    L.block = nwaves * 64;
     L.lds = (int32_t)((int64_t)x * c.K * 4);
     L.k_slice = c.K;
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
@@ -463,15 +474,6 @@ int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, 
     }
     c.P->launches.push_back(L);
     return SDDMM_OK;
-}
-
-int64_t env_i64(const char *name, int64_t dflt)
-{
-    const char *e = getenv(name);
-    if (!e || !*e) return dflt;
-    char *end = nullptr;
-    long long v = strtoll(e, &end, 10);
-    return (end && *end == 0) ? (int64_t)v : dflt;
 }
 
 // Common plan builder from host CSR arrays.  d_*_borrowed != null: the device

@@ -46,7 +46,7 @@ using KernelFn = void (*)(const KArgs);
 // Tile kernel: padded tile-order stream, H tiles in LDS.
 struct TileArgs {
     const int32_t *perm;   // stream position -> sorted position, -1 = padding
-    const int32_t *scol;   // column of each stream position (padding: first column of the tile)
+    const int32_t *scol;   // per stream position: byte offset of the column's H row inside the LDS tile (padding: 0)
     const int32_t *grow;   // row of each group of G consecutive stream positions
     const float *sval;     // values in stream order (padding: 0) or null
     const float *val;      // values in sorted order or null
@@ -63,7 +63,7 @@ using TileFn = void (*)(const TileArgs);
 // want_g > 0: that group size or nothing; 0: the preferred one for K
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
-TileFn tile_kernel(const TileVariant &v, int vmode);
+TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves);  // nwaves: 16, 12 or 8 waves per workgroup
 
 // Panel kernel: rows of W resident in VGPRs, column tiles of H in LDS.
 struct PanelArgs {

@@ -2,7 +2,8 @@
 // LDS, nonzeros streamed in tile order with every (row, tile) run padded to a
 // multiple of G positions.
 //
-// The stream lists S tile by tile (tiles of tile_x columns), rows ascending
+// (scol holds, instead of the column, the byte offset of the column's H row
+// inside the LDS tile.)  The stream lists S tile by tile (tiles of tile_x columns), rows ascending
 // inside a tile.  Each run of one row inside one tile is padded with empty
 // positions to a multiple of G, so a group of G lanes always works on ONE row:
 // there is no per-nonzero row test in the inner loop.  A batch is 64
@@ -70,24 +71,32 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // The loop is software-pipelined by hand and free of branches around loads, so
 // that every wait is for exactly the data needed: while batch b is computed,
 // the index data of batch b+2 and the W row slice of batch b+1 are in flight.
-template <int G, int KPL, int VMODE>
-__global__ __launch_bounds__(kLdsBlock)
+template <int G, int KPL, int VMODE, int NW>
+__global__ __launch_bounds__(NW * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
     extern __shared__ float4 lds_tile[];
-    constexpr int NW = kLdsBlock / 64;
     constexpr int K4 = G * KPL;
+    // Groups that share one 16-lane LDS access phase read the 16-byte pieces of
+    // their rows in different orders (piece j ^ rot instead of j), so that their
+    // reads fall into different banks whenever rows are a multiple of 256 bytes
+    // apart.  NB distinct orders need NB base addresses per row; piece j is then
+    // at base[j % NB] + j*G*16, a compile-time offset.
     constexpr int PHASE_GROUPS = (16 / G) >= 1 ? (16 / G) : 1;
-    constexpr int ROT_MASK = (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL) - 1;
+    constexpr int NB = PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL;
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int l = lane & (G - 1);
-    const int rot = (lane / G) & ROT_MASK;
+    const int rot = (lane / G) & (NB - 1);
 
-    int slot[KPL];
+    int slot[KPL];      // float4 index inside a row of lane's piece j
+    int lane_off[NB];   // byte offset of base t relative to the row start
 #pragma unroll
-    for (int j = 0; j < KPL; ++j) slot[j] = (((j + rot) % KPL) * G + l);
+    for (int j = 0; j < KPL; ++j) slot[j] = (j ^ rot) * G + l;
+#pragma unroll
+    for (int t = 0; t < NB; ++t) lane_off[t] = (l + ((t ^ rot) - t) * G) * 16;
+    const char *lds_bytes = reinterpret_cast<const char *>(lds_tile);
 
     const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W);
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H);
@@ -118,7 +127,7 @@ void sddmm_tile_kernel(const TileArgs a)
             const int rows = min(a.tile_x, a.n_cols - tile_base);
             const float4 *src = H4 + (size_t)tile_base * K4;
             const int n4 = rows * K4;
-            for (int i = threadIdx.x; i < n4; i += kLdsBlock) lds_tile[i] = src[i];
+            for (int i = threadIdx.x; i < n4; i += NW * 64) lds_tile[i] = src[i];
             __syncthreads();
         }
         const int nb = (end - begin + 63) >> 6;
@@ -142,19 +151,25 @@ void sddmm_tile_kernel(const TileArgs a)
 #pragma unroll
             for (int j = 0; j < KPL; ++j) w[j] = wr[slot[j]];
         };
-        auto compute = [&](const float4 (&w)[KPL], const Meta &m, int bi) {
+        // c: this batch's G columns, already broadcast inside the group; cn: the
+        // next batch's, requested here after the last LDS read so that their latency
+        // hides behind the reduction and the store
+        auto compute = [&](const float4 (&w)[KPL], const Meta &m, int bi, const int (&c)[G], int (&cn)[G], int next_col) {
             float v = m.sv;
             if (VMODE == 1) v = a.val[max(m.p, 0)];
             float acc[G];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
-                    const int c_i = group_bcast<G, I>(m.col);
-                    const float4 *hr = lds_tile + (c_i - tile_base) * K4;
+                    const char *base[NB];
+#pragma unroll
+                    for (int t = 0; t < NB; ++t) base[t] = lds_bytes + (c[I] + lane_off[t]);
                     float s = 0.f;
 #pragma unroll
-                    for (int j = 0; j < KPL; ++j) s = dot4(w[j], hr[slot[j]], s);
+                    for (int j = 0; j < KPL; ++j)
+                        s = dot4(w[j], *reinterpret_cast<const float4 *>(base[j % NB] + j * G * 16), s);
                     acc[I] = s;
                 }(), ...);
+                ((void)(cn[I] = group_bcast<G, I>(next_col)), ...);
             }(std::make_integer_sequence<int, G>{});
             transpose_reduce_step<G>(acc, l);
             const int pos = begin + (bi << 6) + lane;
@@ -165,14 +180,18 @@ void sddmm_tile_kernel(const TileArgs a)
         Meta m0 = issue_meta(b0);
         Meta m1 = issue_meta(b0 + 1);
         issue_w(wa, m0.row);
+        int ca[G], cb[G];
+        [&]<int... I>(std::integer_sequence<int, I...>) {
+            ((void)(ca[I] = group_bcast<G, I>(m0.col)), ...);
+        }(std::make_integer_sequence<int, G>{});
         for (int bi = b0; bi < b1; bi += 2) {
             Meta m2 = issue_meta(bi + 2);
             issue_w(wb, m1.row);
-            compute(wa, m0, bi);
+            compute(wa, m0, bi, ca, cb, m1.col);
             if (bi + 1 >= b1) break;
             Meta m3 = issue_meta(bi + 3);
             issue_w(wa, m2.row);
-            compute(wb, m1, bi + 1);
+            compute(wb, m1, bi + 1, cb, ca, m2.col);
             m0 = m2;
             m1 = m3;
         }
@@ -196,12 +215,20 @@ TileVariant pick_tile_variant(int K, int want_g)
     return best;
 }
 
-TileFn tile_kernel(const TileVariant &v, int vmode)
+TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves)
 {
-#define SDDMM_CASE(g, kpl)                                                         \
-    if (v.G == g && v.KPL == kpl)                                                  \
-        return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0>                   \
-             : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1> : (TileFn)sddmm_tile_kernel<g, kpl, 2>;
+#define SDDMM_CASE(g, kpl)                                                                             \
+    if (v.G == g && v.KPL == kpl) {                                                                    \
+        if (nwaves == 16)                                                                              \
+            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 16>                               \
+                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 16> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 16>; \
+        if (nwaves == 12)                                                                              \
+            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 12>                               \
+                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 12> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 12>; \
+        if (nwaves == 8)                                                                               \
+            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 8>                                \
+                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 8> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 8>;   \
+    }
     SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
     SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
 #undef SDDMM_CASE
