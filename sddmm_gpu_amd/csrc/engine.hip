@@ -312,12 +312,12 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
 
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
-int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x, int want_g, sddmm_plan_info *I)
+int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x, int want_g, int ks, sddmm_plan_info *I)
 {
     Launch L;
     L.kind = SDDMM_KERNEL_LDS_TILE;
     L.rows = (int64_t)rows.size();
-    const TileVariant tv = pick_tile_variant(c.K, want_g);
+    const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
     const int nwaves = (int)env_i64("SDDMM_TILE_WAVES", 16);
     L.tfn = tv.G ? tile_kernel(tv, 0, nwaves) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
@@ -352,7 +352,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
             const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
             const int64_t len = T.active_end[s] - b;
             const int32_t tile_base = (int32_t)((int64_t)j * x);
-            const int32_t row_bytes = c.K * 4;
+            const int32_t row_bytes = ks * 4;
             int64_t d = poff[s];
             for (int64_t i = 0; i < len; ++i, ++d) {
                 const int32_t p = T.tiled_ind[b + i];
@@ -384,18 +384,18 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
     if (int rc = c.up(&d_tptr, tptr)) return rc;
     a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.tile_ptr = d_tptr;
     L.sval = d_sval;
-    a.n_tiles = T.n_tiles; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
+    a.n_tiles = T.n_tiles; a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     L.block = nwaves * 64;
-    L.lds = (int32_t)((int64_t)x * c.K * 4);
-    L.k_slice = c.K;
+    L.lds = (int32_t)((int64_t)x * ks * 4);
+    L.k_slice = ks;
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_val, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_noval, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     if (I) {
         I->tile_size_x = x; I->tile_size_y = (int32_t)std::min<int64_t>(c.n_rows, INT32_MAX); I->n_col_tiles = T.n_tiles;
         I->n_row_panels = 1; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
-        I->grid = L.grid; I->block = L.block;
+        I->grid = L.grid; I->block = L.block; I->k_slice = ks;
     }
     c.P->info.padded_positions += np;
     c.P->launches.push_back(L);
@@ -533,34 +533,48 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     const int64_t row_bytes = (int64_t)K * 4;
     const int32_t fit_x = (int32_t)std::min<int64_t>(kLdsMaxBytes / row_bytes, INT32_MAX);  // H rows per LDS tile at full K
     const int ks = (K % 128 == 0) ? 128 : (K % 64 == 0) ? 64 : (K % 32 == 0) ? 32 : 0;    // panel kernel K slice
+    // K elements per launch of the tile kernel: all of K while a row of 128 floats or
+    // less keeps tiles wide; beyond that, slices of 128 (or 64) accumulated into out
+    int kt = 0;
+    if (K <= 128 && pick_tile_variant(K, 0).G) kt = K;
+    else if (K > 128 && K % 128 == 0) kt = 128;
+    else if (K > 128 && K % 64 == 0) kt = 64;
+    else if (pick_tile_variant(K, 0).G) kt = K;
+    {
+        const int64_t o = env_i64("SDDMM_TILE_KSLICE", 0);
+        if (o > 0 && K % o == 0 && pick_tile_variant((int)o, 0).G) kt = (int)o;
+    }
+    const int32_t fit_t = kt ? kLdsMaxBytes / (kt * 4) : 0;  // H rows per LDS tile of the tile kernel
 
     int kernel = want;
     if (kernel == SDDMM_KERNEL_AUTO) kernel = SDDMM_KERNEL_HYBRID;
-    if (kernel == SDDMM_KERNEL_LDS_TILE && (!have_vec || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
+    if (kernel == SDDMM_KERNEL_LDS_TILE && !kt && (!have_vec || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
     if (kernel == SDDMM_KERNEL_PANEL && ks == 0) kernel = SDDMM_KERNEL_ROW_GATHER;
+    if (kernel == SDDMM_KERNEL_HYBRID && !kt) kernel = SDDMM_KERNEL_ROW_GATHER;
 
     I.tile_size_x = (int32_t)std::min<int64_t>(n_cols, INT32_MAX);
     I.tile_size_y = (int32_t)std::min<int64_t>(n_rows, INT32_MAX);
     I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1; I.lanes_per_nnz = 8;
 
     if (kernel == SDDMM_KERNEL_HYBRID) {
-        // Rows are split by length into up to three classes, each with the
-        // kernel whose on-chip reuse pays for it:
-        //   long   (>= long_min nonzeros):  LDS-tile stream; each (row, tile) run is long
-        //          enough to amortise re-reading the W row once per tile
-        //   medium : panel kernel; the W row stays in VGPRs across all tiles
-        //   short  (< short_max nonzeros):  row gather; too few nonzeros per tile for a
-        //          staged H tile to be reused
-        // Column span of a row panel (not n_cols) decides how many tiles a panel sweeps.
-        const PanelVariant pv = ks ? pick_panel_variant(ks) : PanelVariant{0, 0, 0};
-        const int64_t panel_rows = ks ? (int64_t)pv.S * pv.NWAVES * 8 : 1;
+        // Rows are split by length into up to three classes:
+        //   long   tile kernel with the default group size: each (row, tile) run is long
+        //          enough to be padded to that group size at little cost
+        //   medium tile kernel with groups of 4 lanes (less padding on short runs)
+        //   short  row gather: a row has so few nonzeros per column tile that padded
+        //          runs would mostly be padding
+        // How many tiles a row's nonzeros spread over is judged from the column span of
+        // panels of consecutive rows, not from n_cols (a banded matrix spans few tiles).
+        int32_t x = tile_x > 0 ? std::min(tile_x, fit_t) : fit_t;
+        x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
         double span = (double)n_cols;
-        if (!ne.empty()) {  // mean column span of panels of consecutive rows
+        if (!ne.empty()) {
+            const size_t chunk = 512;
             double acc = 0; int64_t cnt = 0;
-            for (size_t b = 0; b < ne.size(); b += (size_t)panel_rows * 16) {  // every 16th panel
-                size_t e = std::min(ne.size(), b + (size_t)panel_rows);
+            for (size_t b = 0; b < ne.size(); b += chunk * 16) {  // every 16th chunk of 512 rows
+                size_t e2 = std::min(ne.size(), b + chunk);
                 int32_t cmin = INT32_MAX, cmax = 0;
-                for (size_t i = b; i < e; ++i) {
+                for (size_t i = b; i < e2; ++i) {
                     cmin = std::min(cmin, col_ind[row_ptr[ne[i]]]);
                     cmax = std::max(cmax, col_ind[row_ptr[ne[i] + 1] - 1]);
                 }
@@ -568,13 +582,14 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
             }
             span = acc / (double)cnt;
         }
-        int32_t xa = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
-        const double tiles_a = std::max(1.0, span / std::max(1, xa));
-        int64_t long_min = (have_vec && fit_x >= 8) ? (int64_t)(16.0 * tiles_a) : INT64_MAX;
-        int64_t short_max = (have_vec && fit_x >= 8) ? (int64_t)std::max(8.0, 2.0 * tiles_a) : INT64_MAX;
-        (void)panel_rows;
+        const double tiles = std::max(1.0, span / std::max(1, x));
+        const int g_long = pick_tile_variant(kt, 0).G;
+        const bool have_g4 = pick_tile_variant(kt, 4).G != 0 && g_long != 4;
+        int64_t long_min = (int64_t)std::max(2.0 * g_long, 2.0 * g_long * tiles);
+        int64_t short_max = (int64_t)std::max(4.0, (have_g4 ? 2.0 : 1.0 * g_long) * tiles);
         long_min = env_i64("SDDMM_LONG_ROW_MIN", long_min);
         short_max = env_i64("SDDMM_SHORT_ROW_MAX", short_max);
+        if (!have_g4) long_min = short_max;
         if (short_max > long_min) short_max = long_min;
         std::vector<int32_t> rl, rm, rs;
         int64_t nl = 0, nm = 0, nsh = 0;
@@ -584,28 +599,38 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
             else if (d >= short_max) { rm.push_back(r); nm += d; }
             else { rs.push_back(r); nsh += d; }
         }
-        // classes too small to fill the machine join a neighbour
-        if (!rm.empty() && (nm * 50 < nnz || (int64_t)rm.size() < 64)) {
-            rs.insert(rs.end(), rm.begin(), rm.end()); nsh += nm; rm.clear(); nm = 0;
+        // staging every H tile must be paid for by the nonzeros that use it
+        const int64_t n_tiles_all = (n_cols + x - 1) / x;
+        const int64_t stage_rows = std::max<int64_t>(n_tiles_all, c.cus) * x;
+        if (nl + nm < 8 * stage_rows) {
+            rs.insert(rs.end(), rl.begin(), rl.end()); rs.insert(rs.end(), rm.begin(), rm.end());
+            nsh += nl + nm; nl = nm = 0; rl.clear(); rm.clear();
             std::sort(rs.begin(), rs.end());
+        }
+        // a small problem is one launch: splitting it only adds launch latency
+        if ((nl || nm) && nnz < 4 * 1000 * 1000) {
+            rl.insert(rl.end(), rm.begin(), rm.end()); rl.insert(rl.end(), rs.begin(), rs.end());
+            nl += nm + nsh; nm = nsh = 0; rm.clear(); rs.clear();
+            std::sort(rl.begin(), rl.end());
+        }
+        // a class too small to fill the machine joins its neighbour
+        if (!rm.empty() && nm * 50 < nnz) {
+            auto &dst = rl.empty() ? rs : rl;
+            dst.insert(dst.end(), rm.begin(), rm.end());
+            (rl.empty() ? nsh : nl) += nm; nm = 0; rm.clear();
+            std::sort(dst.begin(), dst.end());
         }
         if (!rl.empty() && nl * 50 < nnz) {
             auto &dst = rm.empty() ? rs : rm;
             dst.insert(dst.end(), rl.begin(), rl.end());
-            (rm.empty() ? nsh : nm) += nl; rl.clear(); nl = 0;
+            (rm.empty() ? nsh : nm) += nl; nl = 0; rl.clear();
             std::sort(dst.begin(), dst.end());
         }
         sddmm_plan_info scratch{};
-        const bool tile_ok = pick_tile_variant(K, 0).G != 0;
-        if (!rl.empty()) {
-            if (tile_ok) { if (int rc = add_tile(c, rl, rl.size() == ne.size(), xa, (int)env_i64("SDDMM_TILE_G", 0), &I)) return rc; }
-            else if (int rc = add_lds_tile(c, rl, rl.size() == ne.size(), xa, tile_y > 0 ? tile_y : (int32_t)std::min<int64_t>(n_rows, INT32_MAX), &I)) return rc;
-        }
-        if (!rm.empty()) {
-            const bool med_tile = tile_ok && fit_x >= 8 && pick_tile_variant(K, 4).G != 0 && env_i64("SDDMM_MEDIUM_PANEL", 0) == 0;
-            if (med_tile) { if (int rc = add_tile(c, rm, rm.size() == ne.size(), xa, 4, rl.empty() ? &I : &scratch)) return rc; }
-            else if (int rc = add_panel(c, rm, ks, tile_x, tile_y, rl.empty() ? &I : &scratch)) return rc;
-        }
+        if (!rl.empty())
+            if (int rc = add_tile(c, rl, rl.size() == ne.size(), x, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
+        if (!rm.empty())
+            if (int rc = add_tile(c, rm, rm.size() == ne.size(), x, 4, kt, rl.empty() ? &I : &scratch)) return rc;
         if (!rs.empty())
             if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
         I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
@@ -615,13 +640,17 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (int rc = add_panel(c, ne, ks, tile_x, tile_y, &I)) return rc;
         I.kernel = kernel; I.class_nnz[1] = nnz; I.class_rows[1] = (int64_t)ne.size();
     } else if (kernel == SDDMM_KERNEL_LDS_TILE) {
-        int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
-        x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
         int32_t y = tile_y > 0 ? tile_y : (int32_t)std::min<int64_t>(std::max<int64_t>(n_rows, 1), INT32_MAX);
-        if (pick_tile_variant(K, 0).G != 0 && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
-            if (int rc = add_tile(c, ne, true, x, 0, &I)) return rc;
+        if (kt && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
+            int32_t x = tile_x > 0 ? std::min(tile_x, fit_t) : fit_t;
+            x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
+            if (int rc = add_tile(c, ne, true, x, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
             I.tile_size_y = y;
-        } else if (int rc = add_lds_tile(c, ne, true, x, y, &I)) return rc;
+        } else {
+            int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
+            x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
+            if (int rc = add_lds_tile(c, ne, true, x, y, &I)) return rc;
+        }
         I.kernel = kernel; I.class_nnz[0] = nnz; I.class_rows[0] = (int64_t)ne.size();
     } else {
         if (int rc = add_row_gather(c, ne, true)) return rc;
@@ -629,7 +658,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     }
     if (!P->launches.empty() && I.grid == 0) { I.grid = P->launches[0].grid; I.block = P->launches[0].block; I.lds_bytes = P->launches[0].lds; }
     I.n_launches = 0;
-    for (const Launch &L : P->launches) I.n_launches += (L.kind == SDDMM_KERNEL_PANEL) ? K / L.k_slice : 1;
+    for (const Launch &L : P->launches) I.n_launches += (L.k_slice > 0 && L.k_slice < K) ? K / L.k_slice : 1;
     I.device_bytes = c.dev_bytes;
     I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     guard.p = nullptr;
@@ -733,8 +762,12 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
             ta.sval = d_val ? nullptr : L.sval;
             ta.W = d_W; ta.H = d_H; ta.out = d_out;
             const TileFn fn = ta.sval ? L.tfn : (val ? L.tfn_val : L.tfn_noval);
-            hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
-                               (hipStream_t)stream, ta);
+            for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
+                ta.k_off = k_off;
+                ta.accumulate = k_off > 0;
+                hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
+                                   (hipStream_t)stream, ta);
+            }
         } else {
             KArgs a = L.ka;
             a.col_ind = plan->d_col;

@@ -55,6 +55,9 @@ struct TileArgs {
     const int32_t *tile_ptr;  // [n_tiles+1] first stream position of each column tile
     int32_t n_tiles;
     int32_t tile_x, n_cols;
+    int32_t K;           // row length of W and H
+    int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)
+    int32_t accumulate;  // add to out instead of overwriting it
 };
 struct TileVariant {
     int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL

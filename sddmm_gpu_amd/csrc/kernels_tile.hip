@@ -98,8 +98,10 @@ void sddmm_tile_kernel(const TileArgs a)
     for (int t = 0; t < NB; ++t) lane_off[t] = (l + ((t ^ rot) - t) * G) * 16;
     const char *lds_bytes = reinterpret_cast<const char *>(lds_tile);
 
-    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W);
-    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H);
+    // this launch covers K elements [k_off, k_off + 4*K4) of rows that are row_k4 float4 long
+    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
+    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
+    const int row_k4 = a.K >> 2;
 
     // This workgroup's share of the stream: an equal, 64-aligned range of
     // positions, walked tile by tile (usually one or two tiles).
@@ -125,9 +127,12 @@ void sddmm_tile_kernel(const TileArgs a)
             if (!first) __syncthreads();  // everyone is done with the previous tile
             first = false;
             const int rows = min(a.tile_x, a.n_cols - tile_base);
-            const float4 *src = H4 + (size_t)tile_base * K4;
+            const float4 *src = H4 + (size_t)tile_base * row_k4;
             const int n4 = rows * K4;
-            for (int i = threadIdx.x; i < n4; i += NW * 64) lds_tile[i] = src[i];
+            for (int i = threadIdx.x; i < n4; i += NW * 64) {
+                const int r = i / K4, q = i - r * K4;
+                lds_tile[i] = src[(size_t)r * row_k4 + q];
+            }
             __syncthreads();
         }
         const int nb = (end - begin + 63) >> 6;
@@ -147,7 +152,7 @@ void sddmm_tile_kernel(const TileArgs a)
             return m;
         };
         auto issue_w = [&](float4 (&w)[KPL], int row) {
-            const float4 *wr = W4 + (size_t)row * K4;
+            const float4 *wr = W4 + (size_t)row * row_k4;
 #pragma unroll
             for (int j = 0; j < KPL; ++j) w[j] = wr[slot[j]];
         };
@@ -173,7 +178,11 @@ void sddmm_tile_kernel(const TileArgs a)
             }(std::make_integer_sequence<int, G>{});
             transpose_reduce_step<G>(acc, l);
             const int pos = begin + (bi << 6) + lane;
-            if (pos < end && m.p >= 0) a.out[m.p] = acc[0] * v;
+            if (pos < end && m.p >= 0) {
+                float res = acc[0] * v;
+                if (a.accumulate) res += a.out[m.p];
+                a.out[m.p] = res;
+            }
         };
 
         float4 wa[KPL], wb[KPL];
