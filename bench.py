@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """SDDMM benchmark: GFLOP/s (2*nnz*K) and fraction of the HBM roofline, fp32.
 
-One "step" is one sddmm_execute over the whole synthetic matrix, inputs
-resident in HBM.  Default workload: the recommender-ratings shape (480,189 x
-17,770, ~100M nnz, K = 128).  Prints ONE JSON line.
+One "step" is one sddmm_execute over the whole synthetic matrix with indices,
+values, W and H resident in HBM and the output left on the device.  Default
+workload: the recommender-ratings shape (480,189 x 17,770, ~100M nnz, K = 128).
+Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps 20] [--warmup 3] [--config 3] [--K 128]
-                  [--kernel auto|row|lds] [--tile-x X] [--tile-y Y] [--sweep-k] [--no-cpu]
+                  [--kernel auto|row|lds|panel|hybrid] [--tile-x X] [--tile-y Y]
+                  [--no-sweep] [--no-cpu] [--copy-probe]
 """
 import argparse
 import json
@@ -19,6 +21,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
+# the default workload (see profiles/*hbm_traffic*.txt for the runs and the
+# copy-kernel scale factors); None where no such measurement exists.
+MEASURED_TRAFFIC = {}
+
 
 def alg_bytes(nnz, n_rows, K, rows_touched, cols_touched):
     """Compulsory bytes, CSR form: col index + S.val + out per nonzero, the row
@@ -26,30 +33,28 @@ def alg_bytes(nnz, n_rows, K, rows_touched, cols_touched):
     return 12.0 * nnz + 4.0 * (n_rows + 1) + 4.0 * K * (rows_touched + cols_touched)
 
 
-def time_steps(plan, W, H, out, steps, warmup, torch):
+def time_steps(run, steps, warmup, torch):
     stream = torch.cuda.current_stream()
     for _ in range(warmup):
-        plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), stream.cuda_stream)
+        run(stream.cuda_stream)
     torch.cuda.synchronize()
-    # whole timed region (wall clock, synchronised on both sides)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
     for a, b in evs:
-        a.record(stream)
-        plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), stream.cuda_stream)
+        a.record(stream)  # HIP events on the stream the kernels are launched on
+        run(stream.cuda_stream)
         b.record(stream)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    per = sorted(a.elapsed_time(b) for a, b in evs)  # HIP events on the launch stream
+    per = sorted(a.elapsed_time(b) for a, b in evs)
     return wall_ms / steps, sum(per) / len(per), per[len(per) // 2]
 
 
-def cpu_baseline(d, K, torch, budget_s=12.0):
-    """The CPU oracle's OpenMP COO loop (the reference's CPU path restated,
-    with the S.val factor applied) on a bounded leading slice of the same
-    workload, all host threads."""
+def cpu_baseline(d, K, budget_s=12.0):
+    """The CPU oracle's OpenMP COO loop (the reference's CPU path restated, with
+    the S.val factor applied) on a bounded leading slice of the same workload,
+    on all host threads the box grants."""
     from oracle import oracle
-    import numpy as np
     threads = oracle.max_threads()
     W = d["W"].cpu().numpy()
     H = d["H"].cpu().numpy()
@@ -71,7 +76,10 @@ def cpu_baseline(d, K, torch, budget_s=12.0):
         t = run(n)
     gflops = 2.0 * n * K / t / 1e9
     return dict(value=round(gflops, 3), unit="GFLOP/s", cores=threads, kind="port",
-                sample=f"first {n} of {nnz} nonzeros (rows in order), K={K}, best of 2, {t * 1e3:.1f} ms")
+                sample=f"first {n} of {nnz} nonzeros (rows in order), K={K}, best of 2 runs, {t * 1e3:.1f} ms")
+
+
+KERNEL_NAMES = {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid"}
 
 
 def main():
@@ -85,8 +93,10 @@ def main():
     ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds", "panel", "hybrid"])
     ap.add_argument("--tile-x", type=int, default=0)
     ap.add_argument("--tile-y", type=int, default=0)
-    ap.add_argument("--sweep-k", action="store_true", help="also report K = 32, 128, 256, 512")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the K = 32, 128, 256, 512 report")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB device copy (a known-size reference for HBM counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -99,38 +109,36 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL, "hybrid": capi.KERNEL_HYBRID}[args.kernel]
+    kernel = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE,
+              "panel": capi.KERNEL_PANEL, "hybrid": capi.KERNEL_HYBRID}[args.kernel]
     names = {1: "uniform 4096^2 1%", 2: "bag-of-words 1500x12419", 3: "recommender 480189x17770 ~100M nnz",
              4: "R-MAT 2^22 ~200M nnz", 5: "banded 2^20 64/row"}
 
     d = synth.make(args.config, args.scale, device=dev, K=args.K)
     K0 = d["K"]
+    sigma = float(d["W"].std())
 
-    def measure(K):
+    def set_rank(K):
         if K != d["K"]:
             g = torch.Generator(device=dev); g.manual_seed(1000 + K)
-            sigma = float(d["W"].std())
             d["W"] = torch.randn(d["n_rows"], K, generator=g, device=dev) * sigma
             d["H"] = torch.randn(d["n_cols"], K, generator=g, device=dev) * sigma
             d["K"] = K
+
+    def measure(K):
+        set_rank(K)
         plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(),
                                          d["col_ind"].data_ptr(), K, args.tile_x, args.tile_y, kernel)
         info = plan.info()
         out = torch.empty(d["nnz"], device=dev)
-        # the plan holds no values (device CSR): pass S.val at execute
-        stream = torch.cuda.current_stream()
-        val_ptr = d["val"].data_ptr()
-
-        class P:  # binds the value array
-            @staticmethod
-            def execute(_, w, h, o, s):
-                plan.execute(val_ptr, w, h, o, s)
-        wall, mean_ev, med_ev = time_steps(P, d["W"], d["H"], out, args.steps, args.warmup, torch)
+        vp, wp, hp, op = d["val"].data_ptr(), d["W"].data_ptr(), d["H"].data_ptr(), out.data_ptr()
+        wall, mean_ev, med_ev = time_steps(lambda s: plan.execute(vp, wp, hp, op, s), args.steps, args.warmup, torch)
+        prof = plan.execute_profiled(vp, wp, hp, op, torch.cuda.current_stream().cuda_stream)
         flops = 2.0 * d["nnz"] * K
         balg = alg_bytes(d["nnz"], d["n_rows"], K, info["rows_touched"], info["cols_touched"])
         res = dict(K=K, ms_per_step=wall, kernel_ms_mean=mean_ev, kernel_ms_median=med_ev,
                    gflops=flops / (wall * 1e6), alg_bytes=balg, alg_gbps=balg / (mean_ev * 1e6),
-                   frac=balg / (mean_ev * 1e6) / HBM_PEAK_GBPS, info=info, checksum=float(out.double().sum()))
+                   frac=balg / (mean_ev * 1e6) / HBM_PEAK_GBPS, info=info, prof=prof)
         plan.close()
         return res
 
@@ -151,31 +159,36 @@ def main():
         "data": "synthetic",
         "config": {"workload": names[args.config] + (f" (scale {args.scale})" if args.scale != 1.0 else ""),
                    "n_rows": d["n_rows"], "n_cols": d["n_cols"], "nnz": d["nnz"], "K": K0, "seed": d["seed"],
-                   "kernel": {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid"}[info["kernel"]],
-                   "tile_size_x": info["tile_size_x"], "tile_size_y": info["tile_size_y"],
-                   "lanes_per_nnz": info["lanes_per_nnz"], "grid": info["grid"], "block": info["block"],
-                   "lds_bytes": info["lds_bytes"], "n_launches": info["n_launches"],
-                   "class_nnz_lds_panel_row": info["class_nnz"], "class_rows_lds_panel_row": info["class_rows"],
-                   "plan_ms": round(info["plan_ms"], 1)},
+                   "kernel": KERNEL_NAMES[info["kernel"]], "tile_size_x": info["tile_size_x"],
+                   "tile_size_y": info["tile_size_y"], "k_slice": info["k_slice"],
+                   "kernel_launches_per_step": info["n_launches"], "plan_ms": round(info["plan_ms"], 1)},
         "roofline": {"bound": "hbm", "achieved": round(main_res["alg_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(main_res["frac"], 4), "traffic": None,
-                     "alg_bytes_per_launch": main_res["alg_bytes"], "kernel_ms": round(main_res["kernel_ms_mean"], 5)},
+                     "frac": round(main_res["frac"], 4),
+                     "traffic": MEASURED_TRAFFIC.get((args.config, args.scale, K0, args.kernel, args.tile_x, args.tile_y)),
+                     "alg_bytes_per_step": main_res["alg_bytes"], "kernel_ms": round(main_res["kernel_ms_mean"], 5),
+                     "kernels": [{"kernel": KERNEL_NAMES[p["kernel"]], "lanes_per_nnz": p["lanes_per_nnz"],
+                                  "k_slice": p["k_slice"], "launches": p["n_kernel_launches"], "nnz": p["nnz"],
+                                  "rows": p["rows"], "stream_positions": p["stream_positions"],
+                                  "ms": round(p["ms"], 5)} for p in main_res["prof"]]},
     }
-    if args.sweep_k:
+    if not args.no_sweep and args.config == 3:
         sweep = {}
         for K in (32, 128, 256, 512):
             r = main_res if K == K0 else measure(K)
             sweep[str(K)] = {"gflops": round(r["gflops"], 1), "kernel_ms": round(r["kernel_ms_mean"], 4),
                              "hbm_frac": round(r["frac"], 4)}
         line["gflops_by_K"] = sweep
+    if args.copy_probe:
+        n = 1 << 30
+        a = torch.empty(n // 4, device=dev); b = torch.empty_like(a)
+        a.fill_(1.0)
+        torch.cuda.synchronize()
+        b.copy_(a)
+        torch.cuda.synchronize()
+        line["copy_probe_bytes_each_way"] = n
     if not args.no_cpu:
-        if d["K"] != K0:
-            measure_K = K0
-            g = torch.Generator(device=dev); g.manual_seed(1000 + K0)
-            d["W"] = torch.randn(d["n_rows"], K0, generator=g, device=dev) * 0.05
-            d["H"] = torch.randn(d["n_cols"], K0, generator=g, device=dev) * 0.05
-            d["K"] = K0
-        line["cpu_baseline"] = cpu_baseline(d, K0, torch)
+        set_rank(K0)
+        line["cpu_baseline"] = cpu_baseline(d, K0)
     print(json.dumps(line))
 
 

@@ -192,6 +192,24 @@ void sddmm_plan_destroy(sddmm_plan *plan);
 int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
                   float *d_out, void *stream);
 
+/* The same execution with an event after every launch-list entry: fills one
+ * profile per entry (sddmm_plan_launch_count of them) with its wall time on
+ * the device, then returns (synchronises on the last event).  No counterpart
+ * in the reference, which times its whole launch loop with one event pair
+ * (sddmm.cu:93-112); the bench uses it to attribute time to kernel families. */
+typedef struct sddmm_launch_profile {
+    int32_t kernel;            /* SDDMM_KERNEL_ROW_GATHER / LDS_TILE / PANEL */
+    int32_t lanes_per_nnz;
+    int32_t k_slice;           /* K elements per kernel launch */
+    int32_t n_kernel_launches; /* K / k_slice */
+    int64_t nnz, rows;         /* nonzeros and rows this entry covers */
+    int64_t stream_positions;  /* positions walked, padding included */
+    float ms;
+} sddmm_launch_profile;
+int sddmm_plan_launch_count(const sddmm_plan *plan, int32_t *n);
+int sddmm_execute_profiled(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                           float *d_out, void *stream, sddmm_launch_profile *prof, int32_t max_prof);
+
 /* Host-pointer form with the calling convention of the reference's
  * sddmm_GPU(S, tiledS, P, W, H) (sddmm.cu:32): copies W and H to the device,
  * runs the kernels between two events, copies the result back into h_out

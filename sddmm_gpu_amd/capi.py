@@ -37,6 +37,11 @@ class PlanInfo(C.Structure):
         return {f: (list(getattr(self, f)) if f.startswith("class_") else getattr(self, f)) for f, _ in self._fields_}
 
 
+class LaunchProfile(C.Structure):
+    _fields_ = [("kernel", c_int32), ("lanes_per_nnz", c_int32), ("k_slice", c_int32), ("n_kernel_launches", c_int32),
+                ("nnz", c_int64), ("rows", c_int64), ("stream_positions", c_int64), ("ms", c_float)]
+
+
 class TilingView(C.Structure):
     _fields_ = [("tile_size_x", c_int32), ("tile_size_y", c_int32), ("n_col_tiles", c_int32),
                 ("max_active_rows", c_int32), ("nnz", c_int64), ("tile_ptr", POINTER(c_int32)),
@@ -70,6 +75,8 @@ SIGNATURES = {
     "sddmm_plan_get_info": (c_int, [c_void_p, POINTER(PlanInfo)]),
     "sddmm_plan_destroy": (None, [c_void_p]),
     "sddmm_execute": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
+    "sddmm_execute_profiled": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(LaunchProfile), c_int32]),
     "sddmm_gpu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_float)]),
     "sddmm_device_info": (c_int, [POINTER(c_int), c_char_p, c_int]),
 }
@@ -238,6 +245,14 @@ class Plan:
     def execute(self, d_val, d_W, d_H, d_out, stream=0):
         check(lib().sddmm_execute(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
                                   c_void_p(stream or None)))
+
+    def execute_profiled(self, d_val, d_W, d_H, d_out, stream=0):
+        n = c_int32()
+        check(lib().sddmm_plan_launch_count(self.h, byref(n)))
+        prof = (LaunchProfile * max(n.value, 1))()
+        check(lib().sddmm_execute_profiled(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
+                                           c_void_p(stream or None), prof, n.value))
+        return [{f: getattr(prof[i], f) for f, _ in LaunchProfile._fields_} for i in range(n.value)]
 
     def gpu(self, W, H):
         """Host arrays in, host array out (+ kernel-only ms): the calling

@@ -44,7 +44,8 @@ struct Launch {
     TileArgs ta{};
     const float *sval = nullptr;  // the plan's values in stream order (LDS_TILE)
     int32_t grid = 0, block = 0, lds = 0, k_slice = 0;
-    int64_t nnz = 0, rows = 0;
+    int32_t tile_g = 0, gather_g = 8;
+    int64_t nnz = 0, rows = 0, positions = 0;
 };
 
 struct sddmm_plan {
@@ -225,6 +226,7 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
     L.block = kRowGatherBlock;
     L.k_slice = c.K;
     c.P->info.lanes_per_nnz = var.G ? var.G : 8;
+    L.gather_g = var.G ? var.G : 8; L.positions = n;
     c.P->launches.push_back(L);
     return SDDMM_OK;
 }
@@ -398,6 +400,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
         I->grid = L.grid; I->block = L.block; I->k_slice = ks;
     }
     c.P->info.padded_positions += np;
+    L.positions = np; L.tile_g = G;
     c.P->launches.push_back(L);
     return SDDMM_OK;
 }
@@ -608,7 +611,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
             std::sort(rs.begin(), rs.end());
         }
         // a small problem is one launch: splitting it only adds launch latency
-        if ((nl || nm) && nnz < 4 * 1000 * 1000) {
+        if ((nl || nm) && nnz < env_i64("SDDMM_SPLIT_MIN_NNZ", 4 * 1000 * 1000)) {
             rl.insert(rl.end(), rm.begin(), rm.end()); rl.insert(rl.end(), rs.begin(), rs.end());
             nl += nm + nsh; nm = nsh = 0; rm.clear(); rs.clear();
             std::sort(rl.begin(), rl.end());
@@ -735,50 +738,100 @@ int sddmm_plan_get_info(const sddmm_plan *plan, sddmm_plan_info *info)
 
 void sddmm_plan_destroy(sddmm_plan *plan) { delete plan; }
 
+static int check_execute_args(const sddmm_plan *plan, const float *d_W, const float *d_H, float *d_out, const char *who)
+{
+    if (!plan) return fail(SDDMM_ERR_ARG, "%s: plan is NULL", who);
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    if (!d_W || !d_H || !d_out) return fail(SDDMM_ERR_ARG, "%s: NULL device pointer", who);
+    if ((((uintptr_t)d_W | (uintptr_t)d_H) & 15u) && plan->info.K % 4 == 0)
+        return fail(SDDMM_ERR_ARG, "%s: W and H must be 16-byte aligned", who);
+    return SDDMM_OK;
+}
+
+// Issues the kernels of one launch-list entry (one per K slice) on `stream`.
+static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d_val, const float *d_W,
+                         const float *d_H, float *d_out, hipStream_t stream)
+{
+    const sddmm_plan_info &I = plan->info;
+    const float *val = d_val ? d_val : plan->d_val;
+    if (L.kind == SDDMM_KERNEL_PANEL) {
+        PanelArgs pa = L.pa;
+        pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
+        pa.val = val; pa.W = d_W; pa.H = d_H; pa.out = d_out;
+        for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
+            pa.k_off = k_off;
+            pa.accumulate = k_off > 0;
+            hipLaunchKernelGGL(L.pfn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, pa);
+        }
+    } else if (L.tfn) {
+        TileArgs ta = L.ta;
+        ta.val = val;
+        ta.sval = d_val ? nullptr : L.sval;
+        ta.W = d_W; ta.H = d_H; ta.out = d_out;
+        const TileFn fn = ta.sval ? L.tfn : (val ? L.tfn_val : L.tfn_noval);
+        for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
+            ta.k_off = k_off;
+            ta.accumulate = k_off > 0;
+            hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
+        }
+    } else {
+        KArgs a = L.ka;
+        a.col_ind = plan->d_col;
+        a.val = val;
+        a.sval = d_val ? nullptr : L.sval;
+        a.W = d_W; a.H = d_H; a.out = d_out;
+        hipLaunchKernelGGL(L.fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, a);
+    }
+}
+
 int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H, float *d_out,
                   void *stream)
 {
-    if (!plan) return fail(SDDMM_ERR_ARG, "sddmm_execute: plan is NULL");
-    const sddmm_plan_info &I = plan->info;
-    if (I.nnz == 0) return SDDMM_OK;
-    if (!d_W || !d_H || !d_out) return fail(SDDMM_ERR_ARG, "sddmm_execute: NULL device pointer");
-    if ((((uintptr_t)d_W | (uintptr_t)d_H) & 15u) && I.K % 4 == 0)
-        return fail(SDDMM_ERR_ARG, "sddmm_execute: W and H must be 16-byte aligned");
-    const float *val = d_val ? d_val : plan->d_val;
-    for (const Launch &L : plan->launches) {
-        if (L.kind == SDDMM_KERNEL_PANEL) {
-            PanelArgs pa = L.pa;
-            pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
-            pa.val = val; pa.W = d_W; pa.H = d_H; pa.out = d_out;
-            for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
-                pa.k_off = k_off;
-                pa.accumulate = k_off > 0;
-                hipLaunchKernelGGL(L.pfn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
-                                   (hipStream_t)stream, pa);
-            }
-        } else if (L.tfn) {
-            TileArgs ta = L.ta;
-            ta.val = val;
-            ta.sval = d_val ? nullptr : L.sval;
-            ta.W = d_W; ta.H = d_H; ta.out = d_out;
-            const TileFn fn = ta.sval ? L.tfn : (val ? L.tfn_val : L.tfn_noval);
-            for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
-                ta.k_off = k_off;
-                ta.accumulate = k_off > 0;
-                hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
-                                   (hipStream_t)stream, ta);
-            }
-        } else {
-            KArgs a = L.ka;
-            a.col_ind = plan->d_col;
-            a.val = val;
-            a.sval = d_val ? nullptr : L.sval;
-            a.W = d_W; a.H = d_H; a.out = d_out;
-            hipLaunchKernelGGL(L.fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
-                               (hipStream_t)stream, a);
-        }
+    if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute")) return rc;
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream);
+    HIP_TRY(hipGetLastError());
+    return SDDMM_OK;
+}
+
+int sddmm_plan_launch_count(const sddmm_plan *plan, int32_t *n)
+{
+    if (!plan || !n) return fail(SDDMM_ERR_ARG, "sddmm_plan_launch_count: NULL argument");
+    *n = (int32_t)plan->launches.size();
+    return SDDMM_OK;
+}
+
+int sddmm_execute_profiled(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                           float *d_out, void *stream, sddmm_launch_profile *prof, int32_t max_prof)
+{
+    if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute_profiled")) return rc;
+    if (!prof || max_prof < (int32_t)plan->launches.size())
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_profiled: room for %zu profiles needed", plan->launches.size());
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    const size_t n = plan->launches.size();
+    std::vector<hipEvent_t> ev(n + 1, nullptr);
+    struct Ev { std::vector<hipEvent_t> &e; ~Ev() { for (auto x : e) if (x) (void)hipEventDestroy(x); } } guard{ev};
+    for (auto &x : ev) HIP_TRY(hipEventCreate(&x));
+    HIP_TRY(hipEventRecord(ev[0], (hipStream_t)stream));
+    for (size_t i = 0; i < n; ++i) {
+        issue_launch(plan, plan->launches[i], d_val, d_W, d_H, d_out, (hipStream_t)stream);
+        HIP_TRY(hipEventRecord(ev[i + 1], (hipStream_t)stream));
     }
     HIP_TRY(hipGetLastError());
+    HIP_TRY(hipEventSynchronize(ev[n]));
+    for (size_t i = 0; i < n; ++i) {
+        const Launch &L = plan->launches[i];
+        float ms = 0.f;
+        HIP_TRY(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
+        prof[i].kernel = L.kind;
+        prof[i].lanes_per_nnz = L.kind == SDDMM_KERNEL_PANEL ? 8 : (L.tfn ? L.tile_g : L.gather_g);
+        prof[i].k_slice = L.k_slice;
+        prof[i].n_kernel_launches = (L.k_slice > 0 && L.k_slice < plan->info.K) ? plan->info.K / L.k_slice : 1;
+        prof[i].nnz = L.nnz;
+        prof[i].rows = L.rows;
+        prof[i].stream_positions = L.positions;
+        prof[i].ms = ms;
+    }
     return SDDMM_OK;
 }
 

@@ -208,6 +208,7 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     plan through the length thresholds and checks the union of their outputs."""
     monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(long_min))
     monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # split even this small matrix
     d = synth.make(3, 0.02, K=128)
     deg = np.diff(d["row_ptr"].numpy())
     out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID)
