@@ -175,6 +175,16 @@ int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const 
                              const int32_t *d_col_ind, int32_t K, int32_t tile_size_x,
                              int32_t tile_size_y, uint32_t flags, sddmm_plan **out);
 
+/* Gives the plan its own copy of S.val (nnz fp32 in sorted order, device
+ * pointer), laid out the way each of its kernels streams the nonzeros, so
+ * that sddmm_execute(plan, NULL, ...) reads values coalesced.  This is what
+ * sddmm_plan_create does for a host matrix; use it after
+ * sddmm_plan_create_device, or to change the values of a fixed pattern.  Runs
+ * on `stream`; not to be called while an execute of the same plan is in
+ * flight.  The reference uploads the values together with the tiled indices
+ * (tS.vals, util.h:304, sddmm.cu:51).                                        */
+int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream);
+
 int sddmm_plan_get_info(const sddmm_plan *plan, sddmm_plan_info *info);
 void sddmm_plan_destroy(sddmm_plan *plan);
 

@@ -72,6 +72,7 @@ SIGNATURES = {
     "sddmm_plan_create": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_uint32, POINTER(c_void_p)]),
     "sddmm_plan_create_device": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                          c_uint32, POINTER(c_void_p)]),
+    "sddmm_plan_set_values": (c_int, [c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_get_info": (c_int, [c_void_p, POINTER(PlanInfo)]),
     "sddmm_plan_destroy": (None, [c_void_p]),
     "sddmm_execute": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -236,6 +237,9 @@ class Plan:
         check(lib().sddmm_plan_create_device(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K, tile_x,
                                              tile_y, kernel, byref(h)))
         return cls(h, keep)
+
+    def set_values(self, d_val, stream=0):
+        check(lib().sddmm_plan_set_values(self.h, c_void_p(d_val), c_void_p(stream or None)))
 
     def info(self):
         i = PlanInfo()

@@ -42,7 +42,8 @@ struct Launch {
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
-    const float *sval = nullptr;  // the plan's values in stream order (LDS_TILE)
+    float *sval = nullptr;        // the plan's values in stream order (launches that walk a permuted stream)
+    const int32_t *perm = nullptr;  // stream position -> sorted position of that launch (null: identity)
     int32_t grid = 0, block = 0, lds = 0, k_slice = 0;
     int32_t tile_g = 0, gather_g = 8;
     int64_t nnz = 0, rows = 0, positions = 0;
@@ -218,6 +219,7 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
     if (int rc = c.up(&d_bseg, batch_seg)) return rc;
     if (int rc = c.up(&d_bmask, batch_mask)) return rc;
     a.seg_row = d_seg_row; a.perm = d_perm; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
+    L.perm = d_perm;
     a.nnz = (int32_t)n;
     a.chunk = 64 * kRowGatherBatchesPerWave * (kRowGatherBlock / 64);
     a.K = c.K; a.n_cols = (int32_t)c.n_cols; a.tile_x = (int32_t)c.n_cols;
@@ -295,7 +297,7 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     if (int rc = c.up(&d_sval, sval)) return rc;
     a.perm = d_perm; a.seg_row = d_seg_row; a.items = d_items; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
     a.scol = d_scol;
-    L.sval = d_sval;
+    L.sval = d_sval; L.perm = d_perm;
     a.n_items = (int32_t)items.size();
     a.nnz = (int32_t)n; a.K = c.K; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)items.size()));
@@ -314,7 +316,8 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
 
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
-int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x, int want_g, int ks, sddmm_plan_info *I)
+int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_rows, int want_g, int ks,
+             sddmm_plan_info *I)
 {
     Launch L;
     L.kind = SDDMM_KERNEL_LDS_TILE;
@@ -326,67 +329,87 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
     L.tfn_val = tile_kernel(tv, 1, nwaves);
     L.tfn_noval = tile_kernel(tv, 2, nwaves);
     const int G = tv.G;
-    sddmm_tiling T;
-    if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, INT32_MAX, T,
-                              all_rows ? nullptr : rows.data(), (int64_t)rows.size()))
-        return rc;
-    L.nnz = T.nnz;
-    if (T.nnz == 0) return SDDMM_OK;
-    const int64_t n_seg = (int64_t)T.active_end.size();
-    std::vector<int64_t> poff((size_t)n_seg + 1);
-    std::vector<int32_t> seg_tile((size_t)n_seg);
-    poff[0] = 0;
-    for (int32_t j = 0; j < T.n_tiles; ++j)
-        for (int64_t s = T.active_ptr[j]; s < T.active_ptr[j + 1]; ++s) {
-            const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
-            const int64_t len = T.active_end[s] - b;
-            poff[s + 1] = poff[s] + (len + G - 1) / G * G;
-            seg_tile[s] = j;
-        }
-    const int64_t np = poff[n_seg];
-    if (np >= INT32_MAX - 4096) return fail(SDDMM_ERR_RANGE, "plan: padded stream beyond int32 offsets");
-    std::vector<int32_t> perm((size_t)np), scol((size_t)np), grow((size_t)(np / G));
+    L.nnz = list_nnz(c, rows);
+    if (L.nnz == 0) return SDDMM_OK;
+    // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
+    // inside a panel column tile by column tile, inside a tile rows ascending.  A
+    // (panel, tile) pair with nonzeros is a "unit"; workgroups that work on the units of
+    // one panel at the same time share its W rows in L2.
+    if (panel_rows < 1) panel_rows = 1;
+    std::vector<int32_t> perm, scol, grow, unit_ptr, unit_tile;
     std::vector<float> sval;
-    if (c.vals) sval.resize((size_t)np);
-    parallel_ranges(n_seg, 1 << 10, [&](int64_t sb, int64_t se, int) {
-        for (int64_t s = sb; s < se; ++s) {
-            const int32_t j = seg_tile[s];
-            const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
-            const int64_t len = T.active_end[s] - b;
-            const int32_t tile_base = (int32_t)((int64_t)j * x);
-            const int32_t row_bytes = ks * 4;
-            int64_t d = poff[s];
-            for (int64_t i = 0; i < len; ++i, ++d) {
-                const int32_t p = T.tiled_ind[b + i];
-                perm[d] = p;
-                scol[d] = (c.col_ind[p] - tile_base) * row_bytes;  // byte offset of the H row inside the LDS tile
-                if (c.vals) sval[d] = c.vals[p];
+    const size_t guess = (size_t)(L.nnz + L.nnz / 4);
+    perm.reserve(guess); scol.reserve(guess); grow.reserve(guess / G + 1);
+    if (c.vals) sval.reserve(guess);
+    std::vector<int64_t> poff;
+    std::vector<int32_t> seg_tile;
+    int64_t np = 0;
+    int32_t n_tiles_all = 0, n_panels = 0;
+    for (size_t rb = 0; rb < rows.size(); rb += (size_t)panel_rows, ++n_panels) {
+        const int64_t nr = (int64_t)std::min(rows.size() - rb, (size_t)panel_rows);
+        sddmm_tiling T;
+        if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, INT32_MAX, T, rows.data() + rb, nr))
+            return rc;
+        n_tiles_all = T.n_tiles;
+        const int64_t n_seg = (int64_t)T.active_end.size();
+        poff.assign((size_t)n_seg + 1, 0);
+        seg_tile.assign((size_t)n_seg, 0);
+        poff[0] = np;
+        for (int32_t j = 0; j < T.n_tiles; ++j) {
+            if (T.active_ptr[j + 1] > T.active_ptr[j]) {
+                unit_ptr.push_back((int32_t)poff[T.active_ptr[j]]);
+                unit_tile.push_back(j);
             }
-            for (; d < poff[s + 1]; ++d) {
-                perm[d] = -1;
-                scol[d] = 0;
-                if (c.vals) sval[d] = 0.f;
+            for (int64_t s = T.active_ptr[j]; s < T.active_ptr[j + 1]; ++s) {
+                const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
+                const int64_t len = T.active_end[s] - b;
+                poff[s + 1] = poff[s] + (len + G - 1) / G * G;
+                seg_tile[s] = j;
             }
-            for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
         }
-    });
-    // first padded stream position of each tile
-    std::vector<int32_t> tptr((size_t)T.n_tiles + 1);
-    int64_t n_blocks = 0;
-    for (int32_t j = 0; j <= T.n_tiles; ++j) tptr[j] = (int32_t)poff[T.active_ptr[j]];
-    for (int32_t j = 0; j < T.n_tiles; ++j) n_blocks += tptr[j + 1] > tptr[j];
+        const int64_t np_new = poff[n_seg];
+        if (np_new >= INT32_MAX - 4096) return fail(SDDMM_ERR_RANGE, "plan: padded stream beyond int32 offsets");
+        perm.resize((size_t)np_new); scol.resize((size_t)np_new); grow.resize((size_t)(np_new / G));
+        if (c.vals) sval.resize((size_t)np_new);
+        parallel_ranges(n_seg, 1 << 10, [&](int64_t sb, int64_t se, int) {
+            for (int64_t s = sb; s < se; ++s) {
+                const int32_t j = seg_tile[s];
+                const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
+                const int64_t len = T.active_end[s] - b;
+                const int32_t tile_base = (int32_t)((int64_t)j * x);
+                const int32_t row_bytes = ks * 4;
+                int64_t d = poff[s];
+                for (int64_t i = 0; i < len; ++i, ++d) {
+                    const int32_t p = T.tiled_ind[b + i];
+                    perm[d] = p;
+                    scol[d] = (c.col_ind[p] - tile_base) * row_bytes;  // byte offset of the H row inside the LDS tile
+                    if (c.vals) sval[d] = c.vals[p];
+                }
+                for (; d < poff[s + 1]; ++d) {
+                    perm[d] = -1;
+                    scol[d] = 0;
+                    if (c.vals) sval[d] = 0.f;
+                }
+                for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
+            }
+        });
+        np = np_new;
+    }
+    unit_ptr.push_back((int32_t)np);
+    const int64_t n_blocks = (int64_t)unit_tile.size();
     TileArgs &a = L.ta;
     int32_t *d_perm = nullptr, *d_scol = nullptr, *d_grow = nullptr;
     float *d_sval = nullptr;
-    int32_t *d_tptr = nullptr;
+    int32_t *d_uptr = nullptr, *d_utile = nullptr;
     if (int rc = c.up(&d_perm, perm)) return rc;
     if (int rc = c.up(&d_scol, scol)) return rc;
     if (int rc = c.up(&d_grow, grow)) return rc;
     if (int rc = c.up(&d_sval, sval)) return rc;
-    if (int rc = c.up(&d_tptr, tptr)) return rc;
-    a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.tile_ptr = d_tptr;
-    L.sval = d_sval;
-    a.n_tiles = T.n_tiles; a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
+    if (int rc = c.up(&d_uptr, unit_ptr)) return rc;
+    if (int rc = c.up(&d_utile, unit_tile)) return rc;
+    a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.unit_ptr = d_uptr; a.unit_tile = d_utile;
+    L.sval = d_sval; L.perm = d_perm;
+    a.n_units = (int32_t)unit_tile.size(); a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     L.block = nwaves * 64;
     L.lds = (int32_t)((int64_t)x * ks * 4);
@@ -395,8 +418,8 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_t x,
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_val, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_noval, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     if (I) {
-        I->tile_size_x = x; I->tile_size_y = (int32_t)std::min<int64_t>(c.n_rows, INT32_MAX); I->n_col_tiles = T.n_tiles;
-        I->n_row_panels = 1; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
+        I->tile_size_x = x; I->tile_size_y = panel_rows; I->n_col_tiles = n_tiles_all;
+        I->n_row_panels = n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
         I->grid = L.grid; I->block = L.block; I->k_slice = ks;
     }
     c.P->info.padded_positions += np;
@@ -549,6 +572,10 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     }
     const int32_t fit_t = kt ? kLdsMaxBytes / (kt * 4) : 0;  // H rows per LDS tile of the tile kernel
 
+    // row-panel height of the tile kernel's stream: the panel's W slice (y rows of kt floats)
+    // should stay L2-resident while the workgroups sweep the panel's column tiles
+    int32_t y_panel = tile_y > 0 ? tile_y : (kt ? (int32_t)std::max<int64_t>(256, env_i64("SDDMM_PANEL_BYTES", 2 << 20) / (kt * 4)) : 1);
+
     int kernel = want;
     if (kernel == SDDMM_KERNEL_AUTO) kernel = SDDMM_KERNEL_HYBRID;
     if (kernel == SDDMM_KERNEL_LDS_TILE && !kt && (!have_vec || fit_x < 1)) kernel = SDDMM_KERNEL_ROW_GATHER;
@@ -631,9 +658,9 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         }
         sddmm_plan_info scratch{};
         if (!rl.empty())
-            if (int rc = add_tile(c, rl, rl.size() == ne.size(), x, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
+            if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
         if (!rm.empty())
-            if (int rc = add_tile(c, rm, rm.size() == ne.size(), x, 4, kt, rl.empty() ? &I : &scratch)) return rc;
+            if (int rc = add_tile(c, rm, x, y_panel, 4, kt, rl.empty() ? &I : &scratch)) return rc;
         if (!rs.empty())
             if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
         I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
@@ -647,8 +674,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (kt && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_t) : fit_t;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
-            if (int rc = add_tile(c, ne, true, x, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
-            I.tile_size_y = y;
+            if (int rc = add_tile(c, ne, x, tile_y > 0 ? tile_y : y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
         } else {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
@@ -790,6 +816,31 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
     if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute")) return rc;
     if (plan->info.nnz == 0) return SDDMM_OK;
     for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream);
+    HIP_TRY(hipGetLastError());
+    return SDDMM_OK;
+}
+
+int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
+{
+    if (!plan) return fail(SDDMM_ERR_ARG, "sddmm_plan_set_values: plan is NULL");
+    const int64_t nnz = plan->info.nnz;
+    if (nnz == 0) return SDDMM_OK;
+    if (!d_val) return fail(SDDMM_ERR_ARG, "sddmm_plan_set_values: d_val is NULL");
+    if (!plan->d_val) {
+        HIP_TRY(hipMalloc((void **)&plan->d_val, (size_t)nnz * 4));
+        plan->owned.push_back(plan->d_val);
+        plan->info.device_bytes += nnz * 4;
+    }
+    HIP_TRY(hipMemcpyAsync(plan->d_val, d_val, (size_t)nnz * 4, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    for (Launch &L : plan->launches) {
+        if (!L.perm || L.positions <= 0) continue;  // walks S in sorted order: reads d_val directly
+        if (!L.sval) {
+            HIP_TRY(hipMalloc((void **)&L.sval, (size_t)L.positions * 4));
+            plan->owned.push_back(L.sval);
+            plan->info.device_bytes += L.positions * 4;
+        }
+        launch_gather_values(L.perm, plan->d_val, L.sval, L.positions, stream);
+    }
     HIP_TRY(hipGetLastError());
     return SDDMM_OK;
 }

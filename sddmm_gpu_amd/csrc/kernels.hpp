@@ -52,8 +52,9 @@ struct TileArgs {
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;
-    const int32_t *tile_ptr;  // [n_tiles+1] first stream position of each column tile
-    int32_t n_tiles;
+    const int32_t *unit_ptr;   // [n_units+1] first stream position of each (row panel, column tile) unit
+    const int32_t *unit_tile;  // [n_units] the unit's column tile
+    int32_t n_units;
     int32_t tile_x, n_cols;
     int32_t K;           // row length of W and H
     int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)
@@ -67,6 +68,9 @@ using TileFn = void (*)(const TileArgs);
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
 TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves);  // nwaves: 16, 12 or 8 waves per workgroup
+
+// dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
+void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);
 
 // Panel kernel: rows of W resident in VGPRs, column tiles of H in LDS.
 struct PanelArgs {

@@ -17,6 +17,7 @@
 // together by a butterfly of cross-lane exchanges that leaves nonzero i's dot
 // product in lane i, which scales it by S.val and stores it.
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <utility>
 #include "kernels.hpp"
 
@@ -306,6 +307,22 @@ static KernelFn lookup(const Variant &v)
     SDDMM_CASE(16, 6) SDDMM_CASE(16, 8) SDDMM_CASE(32, 6) SDDMM_CASE(32, 8) SDDMM_CASE(64, 6) SDDMM_CASE(64, 8)
 #undef SDDMM_CASE
     return nullptr;
+}
+
+__global__ void gather_values_kernel(const int32_t *__restrict__ perm, const float *__restrict__ src,
+                                     float *__restrict__ dst, int64_t n)
+{
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const int32_t p = perm[i];
+        dst[i] = p >= 0 ? src[p] : 0.f;
+    }
+}
+
+void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream)
+{
+    if (n <= 0) return;
+    const int blocks = (int)std::min<int64_t>((n + 255) / 256, 65536);
+    hipLaunchKernelGGL(gather_values_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, perm, src, dst, n);
 }
 
 KernelFn stream_kernel(const Variant &v, bool lds_tile) { return lds_tile ? lookup<true>(v) : lookup<false>(v); }

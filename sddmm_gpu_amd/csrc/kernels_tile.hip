@@ -105,27 +105,28 @@ void sddmm_tile_kernel(const TileArgs a)
 
     // This workgroup's share of the stream: an equal, 64-aligned range of
     // positions, walked tile by tile (usually one or two tiles).
-    const int64_t total = a.tile_ptr[a.n_tiles];
+    const int64_t total = a.unit_ptr[a.n_units];
     const int lo = (int)(((total * blockIdx.x / gridDim.x) + 63) & ~(int64_t)63);
     const int hi = (blockIdx.x + 1 == gridDim.x) ? (int)total
                                                  : (int)(((total * (blockIdx.x + 1) / gridDim.x) + 63) & ~(int64_t)63);
-    int tile = 0;
-    {   // first tile whose end lies beyond lo
-        int a0 = 0, a1 = a.n_tiles;
+    int unit = 0;
+    {   // first unit whose end lies beyond lo
+        int a0 = 0, a1 = a.n_units;
         while (a0 < a1) {
             const int mid = (a0 + a1) >> 1;
-            if (a.tile_ptr[mid + 1] <= lo) a0 = mid + 1; else a1 = mid;
+            if (a.unit_ptr[mid + 1] <= lo) a0 = mid + 1; else a1 = mid;
         }
-        tile = a0;
+        unit = a0;
     }
-    bool first = true;
-    for (; tile < a.n_tiles && a.tile_ptr[tile] < hi; ++tile) {
-        const int begin = max(lo, a.tile_ptr[tile]), end = min(hi, a.tile_ptr[tile + 1]);
+    int cur_tile = -1;
+    for (; unit < a.n_units && a.unit_ptr[unit] < hi; ++unit) {
+        const int begin = max(lo, a.unit_ptr[unit]), end = min(hi, a.unit_ptr[unit + 1]);
         if (end <= begin) continue;
-        const int tile_base = tile * a.tile_x;
-        {
-            if (!first) __syncthreads();  // everyone is done with the previous tile
-            first = false;
+        const int tile = a.unit_tile[unit];
+        if (tile != cur_tile) {
+            if (cur_tile >= 0) __syncthreads();  // everyone is done with the previous tile
+            cur_tile = tile;
+            const int tile_base = tile * a.tile_x;
             const int rows = min(a.tile_x, a.n_cols - tile_base);
             const float4 *src = H4 + (size_t)tile_base * row_k4;
             const int n4 = rows * K4;

@@ -169,6 +169,28 @@ def test_value_sources_and_host_form(oracle):
         dv = d["val"].to(dev)
         plan.execute(dv.data_ptr(), Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
         check(d, out.cpu().numpy(), oracle)
+        # values handed to the plan once, then changed: execute(NULL) must follow them
+        plan.set_values(dv.data_ptr())
+        plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+        check(d, out.cpu().numpy(), oracle)
+        dv2 = dv * 2.0
+        plan.set_values(dv2.data_ptr())
+        plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+        d2 = dict(d); d2["val"] = d["val"] * 2.0
+        check(d2, out.cpu().numpy(), oracle)
+    # the same on a hybrid plan with all three row classes
+    import os
+    os.environ.update(SDDMM_LONG_ROW_MIN="150", SDDMM_SHORT_ROW_MAX="15", SDDMM_SPLIT_MIN_NNZ="0")
+    try:
+        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, 0, 0,
+                                         capi.KERNEL_HYBRID, keep=(rp, ci))
+    finally:
+        for k in ("SDDMM_LONG_ROW_MIN", "SDDMM_SHORT_ROW_MAX", "SDDMM_SPLIT_MIN_NNZ"):
+            os.environ.pop(k)
+    assert sum(plan.info()["class_nnz"]) == d["nnz"]
+    plan.set_values(dv.data_ptr())
+    plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
+    check(d, out.cpu().numpy(), oracle)
     # (c) host-pointer form with the reference's sddmm_GPU convention
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], rows, cols, vals)
     out_c, ms = S.plan(64).gpu(W, H)
