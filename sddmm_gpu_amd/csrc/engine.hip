@@ -317,13 +317,16 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
 int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_rows, int want_g, int ks,
-             sddmm_plan_info *I)
+             sddmm_plan_info *I, bool gather = false)
 {
+    // gather: the padded stream in plain row order (one tile as wide as S, one panel),
+    // H rows read from global memory instead of an LDS tile
     Launch L;
-    L.kind = SDDMM_KERNEL_LDS_TILE;
+    L.kind = gather ? SDDMM_KERNEL_ROW_GATHER : SDDMM_KERNEL_LDS_TILE;
+    if (gather) { x = (int32_t)std::max<int64_t>(c.n_cols, 1); panel_rows = INT32_MAX; ks = c.K; }
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
-    const int nwaves = (int)env_i64("SDDMM_TILE_WAVES", 16);
+    const int nwaves = gather ? 4 : (int)env_i64("SDDMM_TILE_WAVES", 16);
     L.tfn = tv.G ? tile_kernel(tv, 0, nwaves) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
     L.tfn_val = tile_kernel(tv, 1, nwaves);
@@ -382,7 +385,8 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 for (int64_t i = 0; i < len; ++i, ++d) {
                     const int32_t p = T.tiled_ind[b + i];
                     perm[d] = p;
-                    scol[d] = (c.col_ind[p] - tile_base) * row_bytes;  // byte offset of the H row inside the LDS tile
+                    // byte offset of the H row inside the LDS tile (gather form: the column itself)
+                    scol[d] = gather ? c.col_ind[p] : (c.col_ind[p] - tile_base) * row_bytes;
                     if (c.vals) sval[d] = c.vals[p];
                 }
                 for (; d < poff[s + 1]; ++d) {
@@ -412,8 +416,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     a.n_units = (int32_t)unit_tile.size(); a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     L.block = nwaves * 64;
-    L.lds = (int32_t)((int64_t)x * ks * 4);
+    L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
     L.k_slice = ks;
+    if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_val, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_noval, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
@@ -661,8 +666,15 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
             if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
         if (!rm.empty())
             if (int rc = add_tile(c, rm, x, y_panel, 4, kt, rl.empty() ? &I : &scratch)) return rc;
-        if (!rs.empty())
-            if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
+        if (!rs.empty()) {
+            // short rows: the padded, pipelined kernel reading H from global memory when the
+            // rows are short enough for padding to stay cheap; the plain row gather otherwise
+            const int gg = (int)env_i64("SDDMM_GATHER_G", 8);
+            const bool padded = env_i64("SDDMM_GATHER_PADDED", 1) != 0 && pick_tile_variant(K, gg).G != 0 &&
+                                (!rl.empty() || !rm.empty());
+            if (padded) { if (int rc = add_tile(c, rs, 0, 0, gg, K, nullptr, true)) return rc; }
+            else if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
+        }
         I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
         I.class_nnz[0] = nl; I.class_nnz[1] = nm; I.class_nnz[2] = nsh;
         I.class_rows[0] = (int64_t)rl.size(); I.class_rows[1] = (int64_t)rm.size(); I.class_rows[2] = (int64_t)rs.size();
@@ -682,7 +694,10 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         }
         I.kernel = kernel; I.class_nnz[0] = nnz; I.class_rows[0] = (int64_t)ne.size();
     } else {
-        if (int rc = add_row_gather(c, ne, true)) return rc;
+        const int gg = (int)env_i64("SDDMM_GATHER_G", 0);
+        if (env_i64("SDDMM_ROW_PADDED", 0) != 0 && pick_tile_variant(K, gg).G != 0) {
+            if (int rc = add_tile(c, ne, 0, 0, gg, K, &I, true)) return rc;
+        } else if (int rc = add_row_gather(c, ne, true)) return rc;
         I.kernel = SDDMM_KERNEL_ROW_GATHER; I.class_nnz[2] = nnz; I.class_rows[2] = (int64_t)ne.size();
     }
     if (!P->launches.empty() && I.grid == 0) { I.grid = P->launches[0].grid; I.block = P->launches[0].block; I.lds_bytes = P->launches[0].lds; }

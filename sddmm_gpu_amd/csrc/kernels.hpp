@@ -67,7 +67,8 @@ using TileFn = void (*)(const TileArgs);
 // want_g > 0: that group size or nothing; 0: the preferred one for K
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
-TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves);  // nwaves: 16, 12 or 8 waves per workgroup
+// nwaves: 16, 12 or 8 waves per workgroup with H tiles in LDS; 4: the gather form (H rows from global memory)
+TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves);
 
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);

@@ -71,7 +71,9 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // The loop is software-pipelined by hand and free of branches around loads, so
 // that every wait is for exactly the data needed: while batch b is computed,
 // the index data of batch b+2 and the W row slice of batch b+1 are in flight.
-template <int G, int KPL, int VMODE, int NW>
+// GATHER: no LDS tile; scol holds the column and H rows are read from global
+// memory (the stream is then one unit in row order, for rows too short to tile).
+template <int G, int KPL, int VMODE, int NW, bool GATHER = false>
 __global__ __launch_bounds__(NW * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
@@ -83,7 +85,7 @@ void sddmm_tile_kernel(const TileArgs a)
     // apart.  NB distinct orders need NB base addresses per row; piece j is then
     // at base[j % NB] + j*G*16, a compile-time offset.
     constexpr int PHASE_GROUPS = (16 / G) >= 1 ? (16 / G) : 1;
-    constexpr int NB = PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL;
+    constexpr int NB = GATHER ? 1 : (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL);
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -122,8 +124,8 @@ void sddmm_tile_kernel(const TileArgs a)
     for (; unit < a.n_units && a.unit_ptr[unit] < hi; ++unit) {
         const int begin = max(lo, a.unit_ptr[unit]), end = min(hi, a.unit_ptr[unit + 1]);
         if (end <= begin) continue;
-        const int tile = a.unit_tile[unit];
-        if (tile != cur_tile) {
+        const int tile = GATHER ? 0 : a.unit_tile[unit];
+        if (!GATHER && tile != cur_tile) {
             if (cur_tile >= 0) __syncthreads();  // everyone is done with the previous tile
             cur_tile = tile;
             const int tile_base = tile * a.tile_x;
@@ -166,13 +168,22 @@ void sddmm_tile_kernel(const TileArgs a)
             float acc[G];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
-                    const char *base[NB];
-#pragma unroll
-                    for (int t = 0; t < NB; ++t) base[t] = lds_bytes + (c[I] + lane_off[t]);
                     float s = 0.f;
+                    if constexpr (GATHER) {
+                        const float4 *hr = H4 + (size_t)c[I] * row_k4;
+                        float4 h[KPL];
 #pragma unroll
-                    for (int j = 0; j < KPL; ++j)
-                        s = dot4(w[j], *reinterpret_cast<const float4 *>(base[j % NB] + j * G * 16), s);
+                        for (int j = 0; j < KPL; ++j) h[j] = hr[slot[j]];
+#pragma unroll
+                        for (int j = 0; j < KPL; ++j) s = dot4(w[j], h[j], s);
+                    } else {
+                        const char *base[NB];
+#pragma unroll
+                        for (int t = 0; t < NB; ++t) base[t] = lds_bytes + (c[I] + lane_off[t]);
+#pragma unroll
+                        for (int j = 0; j < KPL; ++j)
+                            s = dot4(w[j], *reinterpret_cast<const float4 *>(base[j % NB] + j * G * 16), s);
+                    }
                     acc[I] = s;
                 }(), ...);
                 ((void)(cn[I] = group_bcast<G, I>(next_col)), ...);
@@ -235,6 +246,9 @@ TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves)
         if (nwaves == 12)                                                                              \
             return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 12>                               \
                  : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 12> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 12>; \
+        if (nwaves == 4)                                                                               \
+            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 4, true>                          \
+                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 4, true> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 4, true>; \
         if (nwaves == 8)                                                                               \
             return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 8>                                \
                  : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 8> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 8>;   \
