@@ -317,7 +317,7 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
 int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_rows, int want_g, int ks,
-             sddmm_plan_info *I, bool gather = false)
+             sddmm_plan_info *I, bool gather = false, bool x_explicit = false)
 {
     // gather: the padded stream in plain row order (one tile as wide as S, one panel),
     // H rows read from global memory instead of an LDS tile
@@ -334,6 +334,27 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
     if (L.nnz == 0) return SDDMM_OK;
+    // Work assignment.  grid2d: every workgroup owns one column tile for good (its H
+    // tile is staged once) and one of `shares` row blocks that are the same for all
+    // tiles, so the workgroups of different tiles read the same W rows at about the same
+    // time and share them in L2.  The tile count is raised to a divisor of the CU count.
+    bool grid2d = !gather && env_i64("SDDMM_TILE_ASSIGN", 1) != 0;
+    int shares = 1;
+    if (grid2d) {
+        const int64_t n_min = (c.n_cols + x - 1) / x;
+        if (n_min <= c.cus) {
+            int64_t n2 = n_min;
+            while (c.cus % n2) ++n2;
+            if (!x_explicit || n2 == n_min) {
+                x = (int32_t)std::max<int64_t>(1, (c.n_cols + n2 - 1) / n2);
+                shares = (int)(c.cus / ((c.n_cols + x - 1) / x));
+            } else {
+                grid2d = false;  // keep the caller's tile width; equal position ranges balance any tile count
+            }
+        }
+        if (grid2d) panel_rows = INT32_MAX;
+    }
+    std::vector<WorkItem> items;
     // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
     // inside a panel column tile by column tile, inside a tile rows ascending.  A
     // (panel, tile) pair with nonzeros is a "unit"; workgroups that work on the units of
@@ -398,6 +419,25 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             }
         });
         np = np_new;
+        if (grid2d) {
+            // row-block boundaries: equal shares of the rows' nonzeros
+            std::vector<int32_t> cut((size_t)shares + 1, INT32_MAX);
+            cut[0] = 0;
+            int64_t acc = 0; int sidx = 1;
+            for (size_t i = 0; i < rows.size() && sidx < shares; ++i) {
+                acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
+                while (sidx < shares && acc >= L.nnz * sidx / shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
+            }
+            std::vector<int32_t> tiles_ne;
+            for (int32_t j = 0; j < T.n_tiles; ++j) if (T.active_ptr[j + 1] > T.active_ptr[j]) tiles_ne.push_back(j);
+            for (int sh = 0; sh < shares; ++sh)
+                for (int32_t j : tiles_ne) {
+                    const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
+                    const int64_t s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
+                    const int64_t s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
+                    items.push_back({(int32_t)poff[s0], (int32_t)poff[s1], 0, j});
+                }
+        }
     }
     unit_ptr.push_back((int32_t)np);
     const int64_t n_blocks = (int64_t)unit_tile.size();
@@ -415,6 +455,12 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     L.sval = d_sval; L.perm = d_perm;
     a.n_units = (int32_t)unit_tile.size(); a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
+    if (grid2d) {
+        WorkItem *d_items = nullptr;
+        if (int rc = c.up(&d_items, items)) return rc;
+        a.items = d_items; a.n_items = (int32_t)items.size();
+        L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)items.size()));
+    }
     L.block = nwaves * 64;
     L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
     L.k_slice = ks;
@@ -663,9 +709,9 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         }
         sddmm_plan_info scratch{};
         if (!rl.empty())
-            if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
+            if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I, false, tile_x > 0)) return rc;
         if (!rm.empty())
-            if (int rc = add_tile(c, rm, x, y_panel, 4, kt, rl.empty() ? &I : &scratch)) return rc;
+            if (int rc = add_tile(c, rm, x, y_panel, 4, kt, rl.empty() ? &I : &scratch, false, tile_x > 0)) return rc;
         if (!rs.empty()) {
             // short rows: the padded, pipelined kernel reading H from global memory when the
             // rows are short enough for padding to stay cheap; the plain row gather otherwise
@@ -686,7 +732,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (kt && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_t) : fit_t;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
-            if (int rc = add_tile(c, ne, x, tile_y > 0 ? tile_y : y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I)) return rc;
+            if (int rc = add_tile(c, ne, x, tile_y > 0 ? tile_y : y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I, false, tile_x > 0)) return rc;
         } else {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));

@@ -55,6 +55,8 @@ struct TileArgs {
     const int32_t *unit_ptr;   // [n_units+1] first stream position of each (row panel, column tile) unit
     const int32_t *unit_tile;  // [n_units] the unit's column tile
     int32_t n_units;
+    const WorkItem *items;     // non-null: workgroup b works on items b, b + grid, ... (each inside one tile)
+    int32_t n_items;
     int32_t tile_x, n_cols;
     int32_t K;           // row length of W and H
     int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)

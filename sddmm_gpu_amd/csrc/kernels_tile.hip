@@ -105,26 +105,36 @@ void sddmm_tile_kernel(const TileArgs a)
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
     const int row_k4 = a.K >> 2;
 
-    // This workgroup's share of the stream: an equal, 64-aligned range of
-    // positions, walked tile by tile (usually one or two tiles).
-    const int64_t total = a.unit_ptr[a.n_units];
-    const int lo = (int)(((total * blockIdx.x / gridDim.x) + 63) & ~(int64_t)63);
-    const int hi = (blockIdx.x + 1 == gridDim.x) ? (int)total
-                                                 : (int)(((total * (blockIdx.x + 1) / gridDim.x) + 63) & ~(int64_t)63);
-    int unit = 0;
-    {   // first unit whose end lies beyond lo
-        int a0 = 0, a1 = a.n_units;
+    // This workgroup's share of the stream: either the items b, b + grid, ... of an item
+    // list (each inside one tile), or an equal, 64-aligned range of positions walked unit by unit.
+    int lo = 0, hi = 0, unit = 0, n_steps;
+    if (a.items) {
+        n_steps = (a.n_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    } else {
+        const int64_t total = a.unit_ptr[a.n_units];
+        lo = (int)(((total * blockIdx.x / gridDim.x) + 63) & ~(int64_t)63);
+        hi = (blockIdx.x + 1 == gridDim.x) ? (int)total
+                                           : (int)(((total * (blockIdx.x + 1) / gridDim.x) + 63) & ~(int64_t)63);
+        int a0 = 0, a1 = a.n_units;  // first unit whose end lies beyond lo
         while (a0 < a1) {
             const int mid = (a0 + a1) >> 1;
             if (a.unit_ptr[mid + 1] <= lo) a0 = mid + 1; else a1 = mid;
         }
         unit = a0;
+        n_steps = 0;
+        for (int u = unit; u < a.n_units && a.unit_ptr[u] < hi; ++u) ++n_steps;
     }
     int cur_tile = -1;
-    for (; unit < a.n_units && a.unit_ptr[unit] < hi; ++unit) {
-        const int begin = max(lo, a.unit_ptr[unit]), end = min(hi, a.unit_ptr[unit + 1]);
+    for (int step = 0; step < n_steps; ++step) {
+        int begin, end, tile;
+        if (a.items) {
+            const WorkItem wi = a.items[blockIdx.x + step * gridDim.x];
+            begin = wi.begin; end = wi.end; tile = wi.tile;
+        } else {
+            begin = max(lo, a.unit_ptr[unit + step]); end = min(hi, a.unit_ptr[unit + step + 1]);
+            tile = GATHER ? 0 : a.unit_tile[unit + step];
+        }
         if (end <= begin) continue;
-        const int tile = GATHER ? 0 : a.unit_tile[unit];
         if (!GATHER && tile != cur_tile) {
             if (cur_tile >= 0) __syncthreads();  // everyone is done with the previous tile
             cur_tile = tile;
