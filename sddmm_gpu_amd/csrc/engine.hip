@@ -338,8 +338,15 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // tile is staged once) and one of `shares` row blocks that are the same for all
     // tiles, so the workgroups of different tiles read the same W rows at about the same
     // time and share them in L2.  The tile count is raised to a divisor of the CU count.
-    bool grid2d = !gather && env_i64("SDDMM_TILE_ASSIGN", 1) != 0;
+    const int assign = (int)env_i64("SDDMM_TILE_ASSIGN", 2);
+    bool grid2d = !gather && assign != 0;
     int shares = 1;
+    // xcd_local: workgroup b runs on die b % 8 (round-robin dispatch), each die has its
+    // own L2.  All column tiles of a row block are then given to workgroups of ONE die,
+    // so that the block's W rows are fetched into one L2 only and the pieces of an
+    // output line, which come from different tiles, meet in that L2 before they leave it.
+    bool xcd_local = false;
+    int xcd_steps = 1;
     if (grid2d) {
         const int64_t n_min = (c.n_cols + x - 1) / x;
         if (n_min <= c.cus) {
@@ -347,7 +354,14 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             while (c.cus % n2) ++n2;
             if (!x_explicit || n2 == n_min) {
                 x = (int32_t)std::max<int64_t>(1, (c.n_cols + n2 - 1) / n2);
-                shares = (int)(c.cus / ((c.n_cols + x - 1) / x));
+                const int64_t nt = (c.n_cols + x - 1) / x;
+                shares = (int)(c.cus / nt);
+                const int64_t per_die = c.cus / 8;
+                if (assign == 2 && c.cus % 8 == 0 && nt == n2 && (n2 % per_die == 0 || per_die % n2 == 0)) {
+                    xcd_local = true;
+                    xcd_steps = (int)std::max<int64_t>(1, n2 / per_die);
+                    shares = 8 * (int)std::max<int64_t>(1, per_die / n2);
+                }
             } else {
                 grid2d = false;  // keep the caller's tile width; equal position ranges balance any tile count
             }
@@ -410,10 +424,12 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                     scol[d] = gather ? c.col_ind[p] : (c.col_ind[p] - tile_base) * row_bytes;
                     if (c.vals) sval[d] = c.vals[p];
                 }
+                // padding repeats the run's last nonzero: the kernel stores every position
+                // without a test, and a repeat stores the same result at the same place
                 for (; d < poff[s + 1]; ++d) {
-                    perm[d] = -1;
-                    scol[d] = 0;
-                    if (c.vals) sval[d] = 0.f;
+                    perm[d] = perm[d - 1];
+                    scol[d] = scol[d - 1];
+                    if (c.vals) sval[d] = sval[d - 1];
                 }
                 for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
             }
@@ -430,13 +446,26 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             }
             std::vector<int32_t> tiles_ne;
             for (int32_t j = 0; j < T.n_tiles; ++j) if (T.active_ptr[j + 1] > T.active_ptr[j]) tiles_ne.push_back(j);
-            for (int sh = 0; sh < shares; ++sh)
-                for (int32_t j : tiles_ne) {
-                    const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
-                    const int64_t s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
-                    const int64_t s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
-                    items.push_back({(int32_t)poff[s0], (int32_t)poff[s1], 0, j});
-                }
+            auto item_of = [&](int sh, int32_t j) -> WorkItem {
+                const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
+                const int64_t s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
+                const int64_t s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
+                return {(int32_t)poff[s0], (int32_t)poff[s1], 0, j};
+            };
+            if (xcd_local) {
+                // items[b + step * cus] is what workgroup b does in its step-th turn
+                const int per_die = c.cus / 8, nt = T.n_tiles;
+                for (int step = 0; step < xcd_steps; ++step)
+                    for (int b = 0; b < c.cus; ++b) {
+                        const int die = b % 8, slot = b / 8;
+                        const int sh = nt >= per_die ? die : die + 8 * (slot / nt);
+                        const int32_t j = nt >= per_die ? slot + per_die * step : slot % nt;
+                        items.push_back(item_of(sh, j));
+                    }
+            } else {
+                for (int sh = 0; sh < shares; ++sh)
+                    for (int32_t j : tiles_ne) items.push_back(item_of(sh, j));
+            }
         }
     }
     unit_ptr.push_back((int32_t)np);

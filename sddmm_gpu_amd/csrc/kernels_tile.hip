@@ -104,6 +104,8 @@ void sddmm_tile_kernel(const TileArgs a)
     const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
     const int row_k4 = a.K >> 2;
+    const int acc_mask = a.accumulate ? -1 : 0;
+    const float *old_base = a.accumulate ? a.out : reinterpret_cast<const float *>(a.perm);
 
     // This workgroup's share of the stream: either the items b, b + grid, ... of an item
     // list (each inside one tile), or an equal, 64-aligned range of positions walked unit by unit.
@@ -151,10 +153,11 @@ void sddmm_tile_kernel(const TileArgs a)
         const int nb = (end - begin + 63) >> 6;
         const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
         if (b0 >= b1) continue;  // (no barrier below this point inside the tile)
+        const int bf = min(b1, (end - begin) >> 6);  // [b0, bf): this wave's batches of 64 whole positions
 
-        // index data of one batch; positions past the item are clamped into it
-        // (their results are discarded), so no load sits behind a branch
-        struct Meta { int row, p, col; float sv; };
+        // index data of one batch; positions past the item are clamped to its last
+        // one (and repeat its work), so no load sits behind a branch
+        struct Meta { int row, p, col; float sv, old; };
         auto issue_meta = [&](int bi) -> Meta {
             const int pc = min(begin + (bi << 6) + lane, end - 1);
             Meta m;
@@ -164,17 +167,23 @@ void sddmm_tile_kernel(const TileArgs a)
             m.sv = (VMODE == 0) ? a.sval[pc] : 1.0f;
             return m;
         };
+        // the previous K slice's partial result, requested one batch ahead of its use
+        // (without accumulation every lane re-reads one word of the index data and drops it)
+        auto issue_old = [&](Meta &m) { m.old = old_base[m.p & acc_mask]; };
         auto issue_w = [&](float4 (&w)[KPL], int row) {
             const float4 *wr = W4 + (size_t)row * row_k4;
 #pragma unroll
             for (int j = 0; j < KPL; ++j) w[j] = wr[slot[j]];
         };
+        float pend_v;  // result of the batch before, not yet stored
+        int pend_p;
+        auto flush = [&]() { a.out[pend_p] = pend_v; };
         // c: this batch's G columns, already broadcast inside the group; cn: the
         // next batch's, requested here after the last LDS read so that their latency
         // hides behind the reduction and the store
-        auto compute = [&](const float4 (&w)[KPL], const Meta &m, int bi, const int (&c)[G], int (&cn)[G], int next_col) {
+        auto compute = [&](const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
             float v = m.sv;
-            if (VMODE == 1) v = a.val[max(m.p, 0)];
+            if (VMODE == 1) v = a.val[m.p];
             float acc[G];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
@@ -199,32 +208,59 @@ void sddmm_tile_kernel(const TileArgs a)
                 ((void)(cn[I] = group_bcast<G, I>(next_col)), ...);
             }(std::make_integer_sequence<int, G>{});
             transpose_reduce_step<G>(acc, l);
-            const int pos = begin + (bi << 6) + lane;
-            if (pos < end && m.p >= 0) {
-                float res = acc[0] * v;
-                if (a.accumulate) res += a.out[m.p];
-                a.out[m.p] = res;
-            }
+            // The store is left to the start of the next batch (flush): issued here it
+            // would sit, unfinished, in front of the loads that batch waits for.  In a
+            // whole batch it needs no predicate: a padding position repeats a nonzero of
+            // its own group and so writes that nonzero's own result a second time.
+            pend_v = fmaf(acc[0], v, a.accumulate ? m.old : 0.f);
+            pend_p = m.p;
         };
 
         float4 wa[KPL], wb[KPL];
-        Meta m0 = issue_meta(b0);
-        Meta m1 = issue_meta(b0 + 1);
-        issue_w(wa, m0.row);
         int ca[G], cb[G];
-        [&]<int... I>(std::integer_sequence<int, I...>) {
-            ((void)(ca[I] = group_bcast<G, I>(m0.col)), ...);
-        }(std::make_integer_sequence<int, G>{});
-        for (int bi = b0; bi < b1; bi += 2) {
-            Meta m2 = issue_meta(bi + 2);
+        if (b0 < bf) {
+            Meta m0 = issue_meta(b0);
+            Meta m1 = issue_meta(b0 + 1);
+            issue_old(m0);
+            issue_w(wa, m0.row);
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                ((void)(ca[I] = group_bcast<G, I>(m0.col)), ...);
+            }(std::make_integer_sequence<int, G>{});
+            Meta m2 = issue_meta(b0 + 2);
+            issue_old(m1);
             issue_w(wb, m1.row);
-            compute(wa, m0, bi, ca, cb, m1.col);
-            if (bi + 1 >= b1) break;
-            Meta m3 = issue_meta(bi + 3);
-            issue_w(wa, m2.row);
-            compute(wb, m1, bi + 1, cb, ca, m2.col);
-            m0 = m2;
-            m1 = m3;
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
+            compute(wa, m0, ca, cb, m1.col);
+            for (int bi = b0 + 1; bi < bf; bi += 2) {
+                flush();
+                Meta m3 = issue_meta(bi + 2);
+                issue_old(m2);
+                issue_w(wa, m2.row);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(wb, m1, cb, ca, m2.col);
+                if (bi + 1 >= bf) break;
+                flush();
+                Meta m4 = issue_meta(bi + 3);
+                issue_old(m3);
+                issue_w(wb, m3.row);
+                __builtin_amdgcn_sched_barrier(0);
+                compute(wa, m2, ca, cb, m3.col);
+                m1 = m3;
+                m2 = m4;
+            }
+            flush();
+        }
+        if (bf < b1) {
+            // the item's last, partial batch: lanes past its end work on the last
+            // position once more and store nothing
+            Meta mt = issue_meta(bf);
+            issue_old(mt);
+            issue_w(wa, mt.row);
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                ((void)(ca[I] = group_bcast<G, I>(mt.col)), ...);
+            }(std::make_integer_sequence<int, G>{});
+            compute(wa, mt, ca, cb, mt.col);
+            if (begin + (bf << 6) + lane < end) flush();
         }
     }
 }
