@@ -6,7 +6,7 @@ values, W and H resident in HBM and the output left on the device.  Default
 workload: the recommender-ratings shape (480,189 x 17,770, ~100M nnz, K = 128).
 Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps 20] [--warmup 3] [--config 3] [--K 128]
+  python bench.py [--gpus 1] [--steps 1000] [--warmup 100] [--config 3] [--K 128]
                   [--kernel auto|row|lds|panel|hybrid] [--tile-x X] [--tile-y Y]
                   [--no-sweep] [--no-cpu] [--copy-probe]
 """
@@ -85,8 +85,10 @@ KERNEL_NAMES = {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid"}
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # a step takes about a millisecond: the defaults time one second of steady state
+    # (the first few dozen steps after an idle period run at lower clocks)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--K", type=int, default=None)

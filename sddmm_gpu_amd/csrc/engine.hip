@@ -323,7 +323,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // H rows read from global memory instead of an LDS tile
     Launch L;
     L.kind = gather ? SDDMM_KERNEL_ROW_GATHER : SDDMM_KERNEL_LDS_TILE;
-    if (gather) { x = (int32_t)std::max<int64_t>(c.n_cols, 1); panel_rows = INT32_MAX; ks = c.K; }
+    if (gather) { x = (int32_t)std::max<int64_t>(c.n_cols, 1); panel_rows = INT32_MAX; }
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
     const int nwaves = gather ? 4 : (int)env_i64("SDDMM_TILE_WAVES", 16);
@@ -334,6 +334,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
     if (L.nnz == 0) return SDDMM_OK;
+    // the kernel addresses W (and, in the gather form, H) rows by 32-bit float4 indices
+    if ((int64_t)c.n_rows * (c.K / 4) > (int64_t)UINT32_MAX || (gather && (int64_t)c.n_cols * (c.K / 4) > (int64_t)UINT32_MAX))
+        return add_row_gather(c, rows, false);
     // Work assignment.  grid2d: every workgroup owns one column tile for good (its H
     // tile is staged once) and one of `shares` row blocks that are the same for all
     // tiles, so the workgroups of different tiles read the same W rows at about the same
@@ -416,12 +419,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 const int64_t len = T.active_end[s] - b;
                 const int32_t tile_base = (int32_t)((int64_t)j * x);
                 const int32_t row_bytes = ks * 4;
+                const uint32_t k4 = (uint32_t)(c.K / 4);  // W and H rows in float4
                 int64_t d = poff[s];
                 for (int64_t i = 0; i < len; ++i, ++d) {
                     const int32_t p = T.tiled_ind[b + i];
                     perm[d] = p;
-                    // byte offset of the H row inside the LDS tile (gather form: the column itself)
-                    scol[d] = gather ? c.col_ind[p] : (c.col_ind[p] - tile_base) * row_bytes;
+                    // byte offset of the H row inside the LDS tile (gather form: index of its first float4 in H)
+                    scol[d] = gather ? (int32_t)((uint32_t)c.col_ind[p] * k4) : (c.col_ind[p] - tile_base) * row_bytes;
                     if (c.vals) sval[d] = c.vals[p];
                 }
                 // padding repeats the run's last nonzero: the kernel stores every position
@@ -431,7 +435,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                     scol[d] = scol[d - 1];
                     if (c.vals) sval[d] = sval[d - 1];
                 }
-                for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = T.active_row[s];
+                for (int64_t g = poff[s] / G; g < poff[s + 1] / G; ++g) grow[g] = (int32_t)((uint32_t)T.active_row[s] * k4);
             }
         });
         np = np_new;
@@ -452,14 +456,32 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 const int64_t s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
                 return {(int32_t)poff[s0], (int32_t)poff[s1], 0, j};
             };
+            // (a work item's positions are addressed by 32-bit byte offsets from its start)
+            if (np_new > (int64_t)1 << 30) return fail(SDDMM_ERR_RANGE, "plan: more than 2^30 stream positions in one tile launch");
             if (xcd_local) {
                 // items[b + step * cus] is what workgroup b does in its step-th turn
                 const int per_die = c.cus / 8, nt = T.n_tiles;
+                // A workgroup with several turns gets tiles of unequal load: the die's
+                // tiles sorted by load are dealt out boustrophedon, heavy with light.
+                std::vector<int32_t> deal((size_t)8 * nt);
+                if (nt >= per_die)
+                    for (int die = 0; die < 8; ++die) {
+                        std::vector<std::pair<int64_t, int32_t>> ld((size_t)nt);
+                        for (int32_t j = 0; j < nt; ++j) {
+                            const WorkItem it = item_of(die, j);
+                            ld[(size_t)j] = {-(int64_t)(it.end - it.begin), j};
+                        }
+                        if (env_i64("SDDMM_TILE_DEAL", 1) != 0) std::sort(ld.begin(), ld.end());
+                        for (int step = 0; step < xcd_steps; ++step)
+                            for (int slot = 0; slot < per_die; ++slot)
+                                deal[(size_t)die * nt + (size_t)step * per_die + slot] =
+                                    ld[(size_t)step * per_die + (step % 2 ? per_die - 1 - slot : slot)].second;
+                    }
                 for (int step = 0; step < xcd_steps; ++step)
                     for (int b = 0; b < c.cus; ++b) {
                         const int die = b % 8, slot = b / 8;
                         const int sh = nt >= per_die ? die : die + 8 * (slot / nt);
-                        const int32_t j = nt >= per_die ? slot + per_die * step : slot % nt;
+                        const int32_t j = nt >= per_die ? deal[(size_t)die * nt + (size_t)step * per_die + slot] : slot % nt;
                         items.push_back(item_of(sh, j));
                     }
             } else {
@@ -739,15 +761,20 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         sddmm_plan_info scratch{};
         if (!rl.empty())
             if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I, false, tile_x > 0)) return rc;
-        if (!rm.empty())
-            if (int rc = add_tile(c, rm, x, y_panel, 4, kt, rl.empty() ? &I : &scratch, false, tile_x > 0)) return rc;
+        if (!rm.empty()) {
+            // (medium rows may use a narrower K slice: wider column tiles, longer runs, more passes)
+            int km = (int)env_i64("SDDMM_MED_KSLICE", kt == 128 ? 64 : kt);
+            if (km <= 0 || km > kt || K % km || !pick_tile_variant(km, 4).G) km = kt;
+            const int32_t xm = km == kt ? x : (int32_t)std::min<int64_t>(kLdsMaxBytes / (km * 4), std::max<int64_t>(n_cols, 1));
+            if (int rc = add_tile(c, rm, xm, y_panel, 4, km, rl.empty() ? &I : &scratch, false, tile_x > 0 && km == kt)) return rc;
+        }
         if (!rs.empty()) {
             // short rows: the padded, pipelined kernel reading H from global memory when the
             // rows are short enough for padding to stay cheap; the plain row gather otherwise
             const int gg = (int)env_i64("SDDMM_GATHER_G", 8);
-            const bool padded = env_i64("SDDMM_GATHER_PADDED", 1) != 0 && pick_tile_variant(K, gg).G != 0 &&
+            const bool padded = env_i64("SDDMM_GATHER_PADDED", 1) != 0 && pick_tile_variant(kt, gg).G != 0 &&
                                 (!rl.empty() || !rm.empty());
-            if (padded) { if (int rc = add_tile(c, rs, 0, 0, gg, K, nullptr, true)) return rc; }
+            if (padded) { if (int rc = add_tile(c, rs, 0, 0, gg, kt, nullptr, true)) return rc; }
             else if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
         }
         I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
@@ -770,8 +797,8 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         I.kernel = kernel; I.class_nnz[0] = nnz; I.class_rows[0] = (int64_t)ne.size();
     } else {
         const int gg = (int)env_i64("SDDMM_GATHER_G", 0);
-        if (env_i64("SDDMM_ROW_PADDED", 0) != 0 && pick_tile_variant(K, gg).G != 0) {
-            if (int rc = add_tile(c, ne, 0, 0, gg, K, &I, true)) return rc;
+        if (env_i64("SDDMM_ROW_PADDED", 0) != 0 && kt && pick_tile_variant(kt, gg).G != 0) {
+            if (int rc = add_tile(c, ne, 0, 0, gg, kt, &I, true)) return rc;
         } else if (int rc = add_row_gather(c, ne, true)) return rc;
         I.kernel = SDDMM_KERNEL_ROW_GATHER; I.class_nnz[2] = nnz; I.class_rows[2] = (int64_t)ne.size();
     }

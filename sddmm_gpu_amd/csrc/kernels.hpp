@@ -45,10 +45,12 @@ using KernelFn = void (*)(const KArgs);
 
 // Tile kernel: padded tile-order stream, H tiles in LDS.
 struct TileArgs {
-    const int32_t *perm;   // stream position -> sorted position, -1 = padding
-    const int32_t *scol;   // per stream position: byte offset of the column's H row inside the LDS tile (padding: 0)
-    const int32_t *grow;   // row of each group of G consecutive stream positions
-    const float *sval;     // values in stream order (padding: 0) or null
+    // (a padding position repeats the last nonzero of its run in perm, scol and sval)
+    const int32_t *perm;   // stream position -> sorted position
+    const int32_t *scol;   // per stream position: byte offset of the column's H row inside the LDS tile;
+                           // gather form: index of the H row's first float4, column * K/4
+    const int32_t *grow;   // per group of G consecutive stream positions: index of the W row's first float4, row * K/4
+    const float *sval;     // values in stream order or null
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;

@@ -104,7 +104,7 @@ void sddmm_tile_kernel(const TileArgs a)
     const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
     const int row_k4 = a.K >> 2;
-    const int acc_mask = a.accumulate ? -1 : 0;
+    const uint32_t acc_mask = a.accumulate ? ~0u : 0u;
     const float *old_base = a.accumulate ? a.out : reinterpret_cast<const float *>(a.perm);
 
     // This workgroup's share of the stream: either the items b, b + grid, ... of an item
@@ -157,26 +157,39 @@ void sddmm_tile_kernel(const TileArgs a)
 
         // index data of one batch; positions past the item are clamped to its last
         // one (and repeat its work), so no load sits behind a branch
-        struct Meta { int row, p, col; float sv, old; };
+        // Index data of one batch.  The arrays are addressed as (uniform base of the
+        // item) + (32-bit byte offset of the lane), the form that needs no per-lane
+        // 64-bit arithmetic; positions past the item are clamped to its last one (and
+        // repeat its work), so no load sits behind a branch.
+        struct Meta { uint32_t wrow, p; int col; float sv, old; };
+        const uint32_t last = (uint32_t)(end - begin - 1);
+        const char *perm_b = reinterpret_cast<const char *>(a.perm + begin);
+        const char *scol_b = reinterpret_cast<const char *>(a.scol + begin);
+        const char *sval_b = reinterpret_cast<const char *>(a.sval + begin);
+        const char *grow_b = reinterpret_cast<const char *>(a.grow + begin / G);
         auto issue_meta = [&](int bi) -> Meta {
-            const int pc = min(begin + (bi << 6) + lane, end - 1);
+            const uint32_t o4 = min((uint32_t)(bi << 6) + (uint32_t)lane, last) << 2;
             Meta m;
-            m.row = a.grow[pc / G];
-            m.p = a.perm[pc];
-            m.col = a.scol[pc];
-            m.sv = (VMODE == 0) ? a.sval[pc] : 1.0f;
+            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + ((o4 / (4 * G)) << 2));
+            m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
+            m.col = *reinterpret_cast<const int *>(scol_b + o4);
+            m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
             return m;
         };
         // the previous K slice's partial result, requested one batch ahead of its use
         // (without accumulation every lane re-reads one word of the index data and drops it)
         auto issue_old = [&](Meta &m) { m.old = old_base[m.p & acc_mask]; };
-        auto issue_w = [&](float4 (&w)[KPL], int row) {
-            const float4 *wr = W4 + (size_t)row * row_k4;
+        // wrow: float4 index of the row's first element in W
+        auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
+            const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
+            wbase[0] = W4 + (wrow + (uint32_t)slot[0]);
 #pragma unroll
-            for (int j = 0; j < KPL; ++j) w[j] = wr[slot[j]];
+            for (int t = 1; t < NB; ++t) wbase[t] = wbase[0] + (slot[t] - slot[0]);
+#pragma unroll
+            for (int j = 0; j < KPL; ++j) w[j] = wbase[j % NB][(j - j % NB) * G];
         };
         float pend_v;  // result of the batch before, not yet stored
-        int pend_p;
+        uint32_t pend_p;
         auto flush = [&]() { a.out[pend_p] = pend_v; };
         // c: this batch's G columns, already broadcast inside the group; cn: the
         // next batch's, requested here after the last LDS read so that their latency
@@ -189,7 +202,7 @@ void sddmm_tile_kernel(const TileArgs a)
                 ((void)[&] {
                     float s = 0.f;
                     if constexpr (GATHER) {
-                        const float4 *hr = H4 + (size_t)c[I] * row_k4;
+                        const float4 *hr = H4 + (uint32_t)c[I];  // scol: float4 index of the H row
                         float4 h[KPL];
 #pragma unroll
                         for (int j = 0; j < KPL; ++j) h[j] = hr[slot[j]];
@@ -222,27 +235,27 @@ void sddmm_tile_kernel(const TileArgs a)
             Meta m0 = issue_meta(b0);
             Meta m1 = issue_meta(b0 + 1);
             issue_old(m0);
-            issue_w(wa, m0.row);
+            issue_w(wa, m0.wrow);
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)(ca[I] = group_bcast<G, I>(m0.col)), ...);
             }(std::make_integer_sequence<int, G>{});
             Meta m2 = issue_meta(b0 + 2);
             issue_old(m1);
-            issue_w(wb, m1.row);
+            issue_w(wb, m1.wrow);
             __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
             compute(wa, m0, ca, cb, m1.col);
             for (int bi = b0 + 1; bi < bf; bi += 2) {
                 flush();
                 Meta m3 = issue_meta(bi + 2);
                 issue_old(m2);
-                issue_w(wa, m2.row);
+                issue_w(wa, m2.wrow);
                 __builtin_amdgcn_sched_barrier(0);
                 compute(wb, m1, cb, ca, m2.col);
                 if (bi + 1 >= bf) break;
                 flush();
                 Meta m4 = issue_meta(bi + 3);
                 issue_old(m3);
-                issue_w(wb, m3.row);
+                issue_w(wb, m3.wrow);
                 __builtin_amdgcn_sched_barrier(0);
                 compute(wa, m2, ca, cb, m3.col);
                 m1 = m3;
@@ -255,7 +268,7 @@ void sddmm_tile_kernel(const TileArgs a)
             // position once more and store nothing
             Meta mt = issue_meta(bf);
             issue_old(mt);
-            issue_w(wa, mt.row);
+            issue_w(wa, mt.wrow);
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)(ca[I] = group_bcast<G, I>(mt.col)), ...);
             }(std::make_integer_sequence<int, G>{});

@@ -226,8 +226,9 @@ def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
 
 @pytest.mark.parametrize("long_min,short_max", [(200, 20), (100, 100), (10 ** 9, 30), (50, 0)])
 def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
-    """Forces the three row classes (LDS-tile / panel / row-gather) of a hybrid
-    plan through the length thresholds and checks the union of their outputs."""
+    """Forces the three row classes (long: tile kernel, medium: tile kernel with
+    groups of 4 lanes in two K slices of 64, short: padded gather) of a hybrid plan
+    through the length thresholds and checks the union of their outputs."""
     monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(long_min))
     monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
     monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # split even this small matrix
@@ -238,5 +239,5 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     assert sum(info["class_nnz"]) == d["nnz"]
     assert sum(info["class_rows"]) == int((deg > 0).sum())
     if long_min == 200 and short_max == 20:
-        assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 3
+        assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 4  # 1 + 2 K slices + 1
         assert info["class_rows"][0] == int((deg >= 200).sum())
