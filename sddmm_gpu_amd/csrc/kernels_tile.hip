@@ -2,20 +2,22 @@
 // LDS, nonzeros streamed in tile order with every (row, tile) run padded to a
 // multiple of G positions.
 //
-// (scol holds, instead of the column, the byte offset of the column's H row
-// inside the LDS tile.)  The stream lists S tile by tile (tiles of tile_x columns), rows ascending
-// inside a tile.  Each run of one row inside one tile is padded with empty
-// positions to a multiple of G, so a group of G lanes always works on ONE row:
-// there is no per-nonzero row test in the inner loop.  A batch is 64
-// consecutive stream positions (one per lane).  While batch b is computed the
-// index data of batch b+1 (original position, column, value, row) and -- if
-// the group's row changes -- its W row slice are already in flight.  For each
-// of its G nonzeros a group reads the H row from LDS in contiguous 16-byte
-// pieces (groups sharing one 16-lane LDS phase start at different pieces, so
-// their reads fall into different banks), multiplies with the W slice held in
-// VGPRs, and a butterfly over the G lanes leaves nonzero i's dot product in
-// lane i, which scales it by S.val and stores it at the nonzero's own
-// position in the output.
+// The stream lists S tile by tile (tiles of tile_x columns), rows ascending
+// inside a tile; scol holds, instead of the column, the byte offset of the
+// column's H row inside the LDS tile.  Each run of one row inside one tile is
+// padded to a multiple of G positions (the padding repeats the run's last
+// nonzero), so a group of G lanes always works on ONE row: there is no
+// per-nonzero row test in the inner loop.  A batch is 64 consecutive stream
+// positions, one per lane.  While batch b is computed, the index data of batch
+// b+2 (output position, LDS offset, value, W row) and the W row slices of
+// batch b+1 are in flight, and the result of batch b-1 is being stored.  Lane l
+// of a group holds slice l of the row's W elements; in step I it reads the same
+// slice of the H row of one of the group's nonzeros from LDS (in 16-byte pieces;
+// the groups sharing one 16-lane LDS phase visit the pieces in different orders,
+// so their reads fall into different banks) and accumulates the partial dot
+// product in register I.  A halving exchange over the G lanes then leaves the
+// whole dot product of nonzero l in lane l, which scales it by S.val and stores
+// it at the nonzero's own position in the output.
 #include <hip/hip_runtime.h>
 #include <utility>
 #include "kernels.hpp"
@@ -33,10 +35,26 @@ __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float ac
     return acc;
 }
 
-template <int G, int I>
-__device__ __forceinline__ int group_bcast(int v)
+// Two ways to walk a group's G nonzeros.
+// XORDER (H tile in LDS, rows a multiple of 256 bytes): lane l works, in its step
+// I, on the group's nonzero I ^ l, so acc[I] of lane l holds lane l's share of
+// nonzero I ^ l.  Every halving step adds to acc[j] the partner lane's acc[j + S],
+// which belongs to the same nonzero; after the last step acc[0] of lane l is the
+// whole dot product of nonzero l.  No lane ever has to choose which of two
+// registers to keep and which to send.  (The lanes of a group then read G
+// different H rows in one instruction: free in LDS, where only banks count.)
+// Otherwise all lanes of a group work on nonzero I in step I and read one
+// contiguous piece of its H row (what global memory wants), and each halving
+// step selects per lane what to keep and what to send.
+template <int G, int I, bool XORDER>
+__device__ __forceinline__ int column_of_step(int v)
 {
-    return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // src = (lane & ~(G-1)) | I
+    if constexpr (XORDER) {
+        if constexpr (I == 0) return v;
+        else return __builtin_amdgcn_ds_swizzle(v, (I << 10) | 0x1f);  // from lane ^ I
+    } else {
+        return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // from lane (lane & ~(G-1)) | I
+    }
 }
 
 template <int S>
@@ -50,18 +68,23 @@ __device__ __forceinline__ float xor_lane(float v)
         return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (S << 10) | 0x1f));
 }
 
-template <int G, int S = G / 2>
+template <int G, bool XORDER, int S = G / 2>
 __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 {
     if constexpr (S >= 1) {
-        const bool upper = (l & S) != 0;
+        if constexpr (XORDER) {
 #pragma unroll
-        for (int j = 0; j < S; ++j) {
-            float keep = upper ? acc[j + S] : acc[j];
-            float send = upper ? acc[j] : acc[j + S];
-            acc[j] = keep + xor_lane<S>(send);
+            for (int j = 0; j < S; ++j) acc[j] += xor_lane<S>(acc[j + S]);
+        } else {
+            const bool upper = (l & S) != 0;
+#pragma unroll
+            for (int j = 0; j < S; ++j) {
+                float keep = upper ? acc[j + S] : acc[j];
+                float send = upper ? acc[j] : acc[j + S];
+                acc[j] = keep + xor_lane<S>(send);
+            }
         }
-        transpose_reduce_step<G, S / 2>(acc, l);
+        transpose_reduce_step<G, XORDER, S / 2>(acc, l);
     }
 }
 
@@ -79,6 +102,7 @@ void sddmm_tile_kernel(const TileArgs a)
 {
     extern __shared__ float4 lds_tile[];
     constexpr int K4 = G * KPL;
+    constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
     // Groups that share one 16-lane LDS access phase read the 16-byte pieces of
     // their rows in different orders (piece j ^ rot instead of j), so that their
     // reads fall into different banks whenever rows are a multiple of 256 bytes
@@ -191,9 +215,8 @@ void sddmm_tile_kernel(const TileArgs a)
         float pend_v;  // result of the batch before, not yet stored
         uint32_t pend_p;
         auto flush = [&]() { a.out[pend_p] = pend_v; };
-        // c: this batch's G columns, already broadcast inside the group; cn: the
-        // next batch's, requested here after the last LDS read so that their latency
-        // hides behind the reduction and the store
+        // c[I]: the column this lane works on in step I; cn: the same for the next batch, requested here after the last LDS
+        // read so that the latency hides behind the reduction
         auto compute = [&](const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
             float v = m.sv;
             if (VMODE == 1) v = a.val[m.p];
@@ -218,9 +241,9 @@ void sddmm_tile_kernel(const TileArgs a)
                     }
                     acc[I] = s;
                 }(), ...);
-                ((void)(cn[I] = group_bcast<G, I>(next_col)), ...);
+                ((void)(cn[I] = column_of_step<G, I, XORDER>(next_col)), ...);
             }(std::make_integer_sequence<int, G>{});
-            transpose_reduce_step<G>(acc, l);
+            transpose_reduce_step<G, XORDER>(acc, l);
             // The store is left to the start of the next batch (flush): issued here it
             // would sit, unfinished, in front of the loads that batch waits for.  In a
             // whole batch it needs no predicate: a padding position repeats a nonzero of
@@ -237,7 +260,7 @@ void sddmm_tile_kernel(const TileArgs a)
             issue_old(m0);
             issue_w(wa, m0.wrow);
             [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)(ca[I] = group_bcast<G, I>(m0.col)), ...);
+                ((void)(ca[I] = column_of_step<G, I, XORDER>(m0.col)), ...);
             }(std::make_integer_sequence<int, G>{});
             Meta m2 = issue_meta(b0 + 2);
             issue_old(m1);
@@ -270,7 +293,7 @@ void sddmm_tile_kernel(const TileArgs a)
             issue_old(mt);
             issue_w(wa, mt.wrow);
             [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)(ca[I] = group_bcast<G, I>(mt.col)), ...);
+                ((void)(ca[I] = column_of_step<G, I, XORDER>(mt.col)), ...);
             }(std::make_integer_sequence<int, G>{});
             compute(wa, mt, ca, cb, mt.col);
             if (begin + (bf << 6) + lane < end) flush();
