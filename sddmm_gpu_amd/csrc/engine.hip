@@ -37,8 +37,8 @@ struct Launch {
     int kind = 0;            // SDDMM_KERNEL_ROW_GATHER / LDS_TILE / PANEL
     KernelFn fn = nullptr;   // stream kernels
     PanelFn pfn = nullptr;   // panel kernel
-    TileFn tfn = nullptr;    // tile kernel (values in stream order)
-    TileFn tfn_val = nullptr, tfn_noval = nullptr;  // same, values in sorted order / no values
+    TileFn tfn = nullptr;        // tile kernel (values in stream order, first K slice); null: not a tile launch
+    TileFn tfns[3][2] = {};      // [values in stream order / in sorted order / none][first K slice / later slices]
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
@@ -314,6 +314,8 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     return SDDMM_OK;
 }
 
+constexpr size_t kStreamSlack = 256;  // readable entries behind a tile stream's arrays
+
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
 int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_rows, int want_g, int ks,
@@ -326,11 +328,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     if (gather) { x = (int32_t)std::max<int64_t>(c.n_cols, 1); panel_rows = INT32_MAX; }
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
-    const int nwaves = gather ? 4 : (int)env_i64("SDDMM_TILE_WAVES", 16);
-    L.tfn = tv.G ? tile_kernel(tv, 0, nwaves) : nullptr;
+    const int nwaves = gather ? 4 : 16;
+    L.tfn = tv.G ? tile_kernel(tv, 0, gather, false) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
-    L.tfn_val = tile_kernel(tv, 1, nwaves);
-    L.tfn_noval = tile_kernel(tv, 2, nwaves);
+    for (int vm = 0; vm < 3; ++vm)
+        for (int ac = 0; ac < 2; ++ac) L.tfns[vm][ac] = tile_kernel(tv, vm, gather, ac != 0);
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
     if (L.nnz == 0) return SDDMM_OK;
@@ -492,6 +494,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     }
     unit_ptr.push_back((int32_t)np);
     const int64_t n_blocks = (int64_t)unit_tile.size();
+    // The kernel requests index data two batches ahead without clamping: past the last
+    // position lie kStreamSlack readable entries whose W row and output position are valid
+    // (zero), because the W slice and, in later K slices, the old output of the batch
+    // after a wave's last one are requested too (and never used).
+    perm.resize((size_t)np + kStreamSlack, 0); scol.resize((size_t)np + kStreamSlack, 0);
+    grow.resize((size_t)(np / G) + kStreamSlack, 0);
+    if (c.vals) sval.resize((size_t)np + kStreamSlack, 0.f);
     TileArgs &a = L.ta;
     int32_t *d_perm = nullptr, *d_scol = nullptr, *d_grow = nullptr;
     float *d_sval = nullptr;
@@ -516,9 +525,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
     L.k_slice = ks;
     if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
-    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
-    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_val, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
-    HIP_TRY(hipFuncSetAttribute((const void *)L.tfn_noval, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    for (int vm = 0; vm < 3; ++vm)
+        for (int ac = 0; ac < 2; ++ac)
+            HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     if (I) {
         I->tile_size_x = x; I->tile_size_y = panel_rows; I->n_col_tiles = n_tiles_all;
         I->n_row_panels = n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
@@ -911,11 +920,10 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.val = val;
         ta.sval = d_val ? nullptr : L.sval;
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
-        const TileFn fn = ta.sval ? L.tfn : (val ? L.tfn_val : L.tfn_noval);
+        const int vm = ta.sval ? 0 : (val ? 1 : 2);
         for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
             ta.k_off = k_off;
-            ta.accumulate = k_off > 0;
-            hipLaunchKernelGGL(fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
+            hipLaunchKernelGGL(L.tfns[vm][k_off > 0], dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
         }
     } else {
         KArgs a = L.ka;
@@ -952,7 +960,7 @@ int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
     for (Launch &L : plan->launches) {
         if (!L.perm || L.positions <= 0) continue;  // walks S in sorted order: reads d_val directly
         if (!L.sval) {
-            HIP_TRY(hipMalloc((void **)&L.sval, (size_t)L.positions * 4));
+            HIP_TRY(hipMalloc((void **)&L.sval, ((size_t)L.positions + kStreamSlack) * 4));  // (see add_tile)
             plan->owned.push_back(L.sval);
             plan->info.device_bytes += L.positions * 4;
         }

@@ -62,7 +62,6 @@ struct TileArgs {
     int32_t tile_x, n_cols;
     int32_t K;           // row length of W and H
     int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)
-    int32_t accumulate;  // add to out instead of overwriting it
 };
 struct TileVariant {
     int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL
@@ -71,8 +70,9 @@ using TileFn = void (*)(const TileArgs);
 // want_g > 0: that group size or nothing; 0: the preferred one for K
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
-// nwaves: 16, 12 or 8 waves per workgroup with H tiles in LDS; 4: the gather form (H rows from global memory)
-TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves);
+// gather: H rows from global memory, 4 waves per workgroup (otherwise H tiles in LDS, 16 waves)
+// accumulate: out += instead of out = (K slices after the first)
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate);
 
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);

@@ -26,6 +26,8 @@ using namespace sddmm;
 
 namespace {
 
+typedef float vec4f __attribute__((ext_vector_type(4)));  // a plain vector: loadable through an LDS-qualified pointer
+
 __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float acc)
 {
     acc = fmaf(a.x, b.x, acc);
@@ -46,26 +48,74 @@ __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float ac
 // Otherwise all lanes of a group work on nonzero I in step I and read one
 // contiguous piece of its H row (what global memory wants), and each halving
 // step selects per lane what to keep and what to send.
+// v of lane (lane ^ X).  Distances below 8 are built from DPP lane selects (VALU,
+// and the compiler folds them into the add that uses the value): the LDS pipe, which
+// a ds_swizzle would occupy, is what the H-tile reads need.
+template <int X>
+__device__ __forceinline__ int from_lane_xor(int v)
+{
+    constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kQuadXor3 = 0x1B, kHalfMirror = 0x141;  // dpp_ctrl
+    if constexpr (X == 0) return v;
+    else if constexpr (X == 1) return __builtin_amdgcn_mov_dpp(v, kQuadXor1, 0xf, 0xf, true);
+    else if constexpr (X == 2) return __builtin_amdgcn_mov_dpp(v, kQuadXor2, 0xf, 0xf, true);
+    else if constexpr (X == 3) return __builtin_amdgcn_mov_dpp(v, kQuadXor3, 0xf, 0xf, true);
+    else if constexpr (X == 7) return __builtin_amdgcn_mov_dpp(v, kHalfMirror, 0xf, 0xf, true);  // lane ^ 7 inside 8 lanes
+    else if constexpr (X < 8)  // lane ^ X = (lane ^ 7) ^ (X ^ 7)
+        return __builtin_amdgcn_mov_dpp(__builtin_amdgcn_mov_dpp(v, kHalfMirror, 0xf, 0xf, true),
+                                        X == 4 ? kQuadXor3 : X == 5 ? kQuadXor2 : kQuadXor1, 0xf, 0xf, true);
+    else return __builtin_amdgcn_ds_swizzle(v, (X << 10) | 0x1f);
+}
+
 template <int G, int I, bool XORDER>
 __device__ __forceinline__ int column_of_step(int v)
 {
-    if constexpr (XORDER) {
-        if constexpr (I == 0) return v;
-        else return __builtin_amdgcn_ds_swizzle(v, (I << 10) | 0x1f);  // from lane ^ I
+    if constexpr (XORDER) return from_lane_xor<I>(v);
+    else return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // from lane (lane & ~(G-1)) | I
+}
+
+// out[I] = (col of the lane this lane serves in step I) + base, for all G steps.
+// With the lane-permuted order and G = 8 or 4 each is ONE v_add_u32 with a DPP lane
+// select on its first operand (plus one v_mov for the half-mirrored copy that steps
+// 4-6 start from).  Written out because the compiler, left alone, keeps the select
+// and the add apart.  Plain VALU instructions only; the leading s_nop covers the two
+// wait states a DPP read needs after a VALU write of the same register.
+template <int G, bool XORDER>
+__device__ __forceinline__ void columns_of_steps(int col, int base, int (&out)[G])
+{
+    if constexpr (XORDER && G == 8) {
+        int hm;
+        out[0] = col + base;
+        asm("s_nop 1\n\t"
+            "v_mov_b32_dpp %[hm], %[c] row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r1], %[c], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r2], %[c], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r3], %[c], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r7], %[c], %[b] row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r4], %[hm], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r5], %[hm], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r6], %[hm], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+            : [hm] "=&v"(hm), [r1] "=&v"(out[1]), [r2] "=&v"(out[2]), [r3] "=&v"(out[3]), [r4] "=&v"(out[4]),
+              [r5] "=&v"(out[5]), [r6] "=&v"(out[6]), [r7] "=&v"(out[7])
+            : [c] "v"(col), [b] "v"(base));
+    } else if constexpr (XORDER && G == 4) {
+        out[0] = col + base;
+        asm("s_nop 1\n\t"
+            "v_add_u32_dpp %[r1], %[c], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r2], %[c], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+            "v_add_u32_dpp %[r3], %[c], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1"
+            : [r1] "=&v"(out[1]), [r2] "=&v"(out[2]), [r3] "=&v"(out[3])
+            : [c] "v"(col), [b] "v"(base));
     } else {
-        return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // from lane (lane & ~(G-1)) | I
+        [&]<int... I>(std::integer_sequence<int, I...>) {
+            ((void)(out[I] = column_of_step<G, I, XORDER>(col) + base), ...);
+        }(std::make_integer_sequence<int, G>{});
     }
 }
 
 template <int S>
 __device__ __forceinline__ float xor_lane(float v)
 {
-    if constexpr (S == 1)
-        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
-    else if constexpr (S == 2)
-        return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
-    else
-        return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (S << 10) | 0x1f));
+    return __int_as_float(from_lane_xor<S>(__float_as_int(v)));
 }
 
 template <int G, bool XORDER, int S = G / 2>
@@ -96,7 +146,7 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // the index data of batch b+2 and the W row slice of batch b+1 are in flight.
 // GATHER: no LDS tile; scol holds the column and H rows are read from global
 // memory (the stream is then one unit in row order, for rows too short to tile).
-template <int G, int KPL, int VMODE, int NW, bool GATHER = false>
+template <int G, int KPL, int VMODE, int NW, bool GATHER, bool ACC>
 __global__ __launch_bounds__(NW * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
@@ -122,14 +172,22 @@ void sddmm_tile_kernel(const TileArgs a)
     for (int j = 0; j < KPL; ++j) slot[j] = (j ^ rot) * G + l;
 #pragma unroll
     for (int t = 0; t < NB; ++t) lane_off[t] = (l + ((t ^ rot) - t) * G) * 16;
-    const char *lds_bytes = reinterpret_cast<const char *>(lds_tile);
+    // LDS addresses are kept as 32-bit integers: the address of this lane's first piece of
+    // an H row is (the row's offset in the tile) + lane_base0, added as soon as the offset arrives
+    using lds_f4_ptr = const __attribute__((address_space(3))) vec4f *;
+    const int lds_base = (int)(uint32_t)(uintptr_t)(lds_f4_ptr)reinterpret_cast<const vec4f *>(lds_tile);
+    const int lane_base0 = GATHER ? 0 : lds_base + lane_off[0];
+    int base_step[NB];  // base t of a row = base 0 + base_step[t]
+#pragma unroll
+    for (int t = 0; t < NB; ++t) {
+        base_step[t] = lane_off[t] - lane_off[0];
+        asm("" : "+v"(base_step[t]));  // one register, not an expression to be re-associated with each use
+    }
 
     // this launch covers K elements [k_off, k_off + 4*K4) of rows that are row_k4 float4 long
     const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
     const int row_k4 = a.K >> 2;
-    const uint32_t acc_mask = a.accumulate ? ~0u : 0u;
-    const float *old_base = a.accumulate ? a.out : reinterpret_cast<const float *>(a.perm);
 
     // This workgroup's share of the stream: either the items b, b + grid, ... of an item
     // list (each inside one tile), or an equal, 64-aligned range of positions walked unit by unit.
@@ -183,26 +241,41 @@ void sddmm_tile_kernel(const TileArgs a)
         // one (and repeat its work), so no load sits behind a branch
         // Index data of one batch.  The arrays are addressed as (uniform base of the
         // item) + (32-bit byte offset of the lane), the form that needs no per-lane
-        // 64-bit arithmetic; positions past the item are clamped to its last one (and
-        // repeat its work), so no load sits behind a branch.
+        // 64-bit arithmetic, and no load sits behind a branch.
         struct Meta { uint32_t wrow, p; int col; float sv, old; };
         const uint32_t last = (uint32_t)(end - begin - 1);
         const char *perm_b = reinterpret_cast<const char *>(a.perm + begin);
         const char *scol_b = reinterpret_cast<const char *>(a.scol + begin);
         const char *sval_b = reinterpret_cast<const char *>(a.sval + begin);
         const char *grow_b = reinterpret_cast<const char *>(a.grow + begin / G);
-        auto issue_meta = [&](int bi) -> Meta {
-            const uint32_t o4 = min((uint32_t)(bi << 6) + (uint32_t)lane, last) << 2;
+        // Steady state: batches are requested in order, two ahead of the one computed,
+        // with running offsets and no clamp (the batch after a wave's last one is
+        // requested and dropped; the arrays have readable slack behind the last position).
+        uint32_t o4 = ((uint32_t)(b0 << 6) + (uint32_t)lane) << 2;         // perm, scol, sval
+        uint32_t og = (((uint32_t)(b0 << 6) + (uint32_t)lane) / G) << 2;   // grow
+        auto issue_meta = [&]() -> Meta {
             Meta m;
-            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + ((o4 / (4 * G)) << 2));
+            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + og);
             m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
             m.col = *reinterpret_cast<const int *>(scol_b + o4);
             m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
+            o4 += 256;
+            og += 256 / G;
             return m;
         };
-        // the previous K slice's partial result, requested one batch ahead of its use
-        // (without accumulation every lane re-reads one word of the index data and drops it)
-        auto issue_old = [&](Meta &m) { m.old = old_base[m.p & acc_mask]; };
+        // an item's last, partial batch: positions past the end are clamped to the last one
+        auto issue_meta_tail = [&](int bi) -> Meta {
+            const uint32_t t4 = min((uint32_t)(bi << 6) + (uint32_t)lane, last) << 2;
+            Meta m;
+            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + ((t4 / (4 * G)) << 2));
+            m.p = *reinterpret_cast<const uint32_t *>(perm_b + t4);
+            m.col = *reinterpret_cast<const int *>(scol_b + t4);
+            m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
+            return m;
+        };
+        // ACC (K slices after the first): the previous slices' partial result, requested
+        // one batch ahead of its use
+        auto issue_old = [&](Meta &m) { m.old = ACC ? a.out[m.p] : 0.f; };
         // wrow: float4 index of the row's first element in W
         auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
             const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
@@ -215,7 +288,8 @@ void sddmm_tile_kernel(const TileArgs a)
         float pend_v;  // result of the batch before, not yet stored
         uint32_t pend_p;
         auto flush = [&]() { a.out[pend_p] = pend_v; };
-        // c[I]: the column this lane works on in step I; cn: the same for the next batch, requested here after the last LDS
+        // c[I]: where the H row this lane works on in step I starts (LDS: byte address of
+        // this lane's first piece; gather form: float4 index of the row); cn: the same for the next batch, requested here after the last LDS
         // read so that the latency hides behind the reduction
         auto compute = [&](const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
             float v = m.sv;
@@ -232,51 +306,52 @@ void sddmm_tile_kernel(const TileArgs a)
 #pragma unroll
                         for (int j = 0; j < KPL; ++j) s = dot4(w[j], h[j], s);
                     } else {
-                        const char *base[NB];
+                        int base[NB];  // c[I] is base 0 already
+                        base[0] = c[I];
 #pragma unroll
-                        for (int t = 0; t < NB; ++t) base[t] = lds_bytes + (c[I] + lane_off[t]);
+                        for (int t = 1; t < NB; ++t) base[t] = c[I] + base_step[t];
 #pragma unroll
-                        for (int j = 0; j < KPL; ++j)
-                            s = dot4(w[j], *reinterpret_cast<const float4 *>(base[j % NB] + j * G * 16), s);
+                        for (int j = 0; j < KPL; ++j) {
+                            const vec4f h = *(lds_f4_ptr)(uintptr_t)(uint32_t)(base[j % NB] + j * G * 16);
+                            s = dot4(w[j], make_float4(h.x, h.y, h.z, h.w), s);
+                        }
                     }
                     acc[I] = s;
                 }(), ...);
-                ((void)(cn[I] = column_of_step<G, I, XORDER>(next_col)), ...);
             }(std::make_integer_sequence<int, G>{});
+            columns_of_steps<G, XORDER>(next_col, lane_base0, cn);
             transpose_reduce_step<G, XORDER>(acc, l);
             // The store is left to the start of the next batch (flush): issued here it
             // would sit, unfinished, in front of the loads that batch waits for.  In a
             // whole batch it needs no predicate: a padding position repeats a nonzero of
             // its own group and so writes that nonzero's own result a second time.
-            pend_v = fmaf(acc[0], v, a.accumulate ? m.old : 0.f);
+            pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
             pend_p = m.p;
         };
 
         float4 wa[KPL], wb[KPL];
         int ca[G], cb[G];
         if (b0 < bf) {
-            Meta m0 = issue_meta(b0);
-            Meta m1 = issue_meta(b0 + 1);
+            Meta m0 = issue_meta();
+            Meta m1 = issue_meta();
             issue_old(m0);
             issue_w(wa, m0.wrow);
-            [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)(ca[I] = column_of_step<G, I, XORDER>(m0.col)), ...);
-            }(std::make_integer_sequence<int, G>{});
-            Meta m2 = issue_meta(b0 + 2);
+            columns_of_steps<G, XORDER>(m0.col, lane_base0, ca);
+            Meta m2 = issue_meta();
             issue_old(m1);
             issue_w(wb, m1.wrow);
             __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
             compute(wa, m0, ca, cb, m1.col);
             for (int bi = b0 + 1; bi < bf; bi += 2) {
                 flush();
-                Meta m3 = issue_meta(bi + 2);
+                Meta m3 = issue_meta();
                 issue_old(m2);
                 issue_w(wa, m2.wrow);
                 __builtin_amdgcn_sched_barrier(0);
                 compute(wb, m1, cb, ca, m2.col);
                 if (bi + 1 >= bf) break;
                 flush();
-                Meta m4 = issue_meta(bi + 3);
+                Meta m4 = issue_meta();
                 issue_old(m3);
                 issue_w(wb, m3.wrow);
                 __builtin_amdgcn_sched_barrier(0);
@@ -289,12 +364,10 @@ void sddmm_tile_kernel(const TileArgs a)
         if (bf < b1) {
             // the item's last, partial batch: lanes past its end work on the last
             // position once more and store nothing
-            Meta mt = issue_meta(bf);
+            Meta mt = issue_meta_tail(bf);
             issue_old(mt);
             issue_w(wa, mt.wrow);
-            [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)(ca[I] = column_of_step<G, I, XORDER>(mt.col)), ...);
-            }(std::make_integer_sequence<int, G>{});
+            columns_of_steps<G, XORDER>(mt.col, lane_base0, ca);
             compute(wa, mt, ca, cb, mt.col);
             if (begin + (bf << 6) + lane < end) flush();
         }
@@ -318,26 +391,20 @@ TileVariant pick_tile_variant(int K, int want_g)
     return best;
 }
 
-TileFn tile_kernel(const TileVariant &v, int vmode, int nwaves)
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate)
 {
-#define SDDMM_CASE(g, kpl)                                                                             \
-    if (v.G == g && v.KPL == kpl) {                                                                    \
-        if (nwaves == 16)                                                                              \
-            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 16>                               \
-                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 16> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 16>; \
-        if (nwaves == 12)                                                                              \
-            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 12>                               \
-                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 12> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 12>; \
-        if (nwaves == 4)                                                                               \
-            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 4, true>                          \
-                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 4, true> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 4, true>; \
-        if (nwaves == 8)                                                                               \
-            return vmode == 0 ? (TileFn)sddmm_tile_kernel<g, kpl, 0, 8>                                \
-                 : vmode == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, 1, 8> : (TileFn)sddmm_tile_kernel<g, kpl, 2, 8>;   \
-    }
+#define SDDMM_PICK(g, kpl, vm)                                                                              \
+    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, true>                            \
+                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
+            : (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, 16, false, true>                          \
+                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 16, false, false>))
+#define SDDMM_CASE(g, kpl)                                                                                  \
+    if (v.G == g && v.KPL == kpl)                                                                           \
+        return vmode == 0 ? SDDMM_PICK(g, kpl, 0) : vmode == 1 ? SDDMM_PICK(g, kpl, 1) : SDDMM_PICK(g, kpl, 2);
     SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
     SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
 #undef SDDMM_CASE
+#undef SDDMM_PICK
     return nullptr;
 }
 

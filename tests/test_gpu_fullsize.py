@@ -13,20 +13,23 @@ from sddmm_gpu_amd import capi, synth
 pytestmark = pytest.mark.gpu
 
 
-def run(d, kernel, W=None):
+def run(d, kernel, W=None, plan_values=False):
     dev = d["val"].device
     plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(), d["col_ind"].data_ptr(),
                                      d["K"], 0, 0, kernel)
     out = torch.full((d["nnz"],), float("nan"), device=dev)
     W = d["W"] if W is None else W
-    plan.execute(d["val"].data_ptr(), W.data_ptr(), d["H"].data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    stream = torch.cuda.current_stream().cuda_stream
+    if plan_values:  # S.val handed to the plan once (what bench.py times) instead of passed per execute
+        plan.set_values(d["val"].data_ptr(), stream)
+    plan.execute(0 if plan_values else d["val"].data_ptr(), W.data_ptr(), d["H"].data_ptr(), out.data_ptr(), stream)
     torch.cuda.synchronize()
     info = plan.info()
     plan.close()
     return out, info
 
 
-@pytest.mark.parametrize("cfg,K", [(3, 128), (4, 64), (5, 512)])
+@pytest.mark.parametrize("cfg,K", [(3, 128), (3, 256), (4, 64), (5, 512)])
 def test_full_size(oracle, cfg, K):
     dev = torch.device("cuda:0")
     d = synth.make(cfg, 1.0, device=dev, K=K)
@@ -52,6 +55,11 @@ def test_full_size(oracle, cfg, K):
     rep = parity_report(out[idx].cpu().numpy(), cpu, K, absp)
     assert rep["violations"] == 0, rep
     del W, H
+
+    # (1b) values kept by the plan in stream order: the same arithmetic, so the same bits
+    outp, _ = run(d, capi.KERNEL_AUTO, plan_values=True)
+    assert torch.equal(outp, out)
+    del outp
 
     # (2) scaling W by a power of two scales every output exactly
     out4, _ = run(d, capi.KERNEL_AUTO, W=d["W"] * 4.0)
