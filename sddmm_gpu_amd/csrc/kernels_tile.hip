@@ -40,9 +40,9 @@ __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float ac
 // Two ways to walk a group's G nonzeros.
 // XORDER (H tile in LDS, rows a multiple of 256 bytes): lane l works, in its step
 // I, on the group's nonzero I ^ l, so acc[I] of lane l holds lane l's share of
-// nonzero I ^ l.  Every halving step adds to acc[j] the partner lane's acc[j + S],
-// which belongs to the same nonzero; after the last step acc[0] of lane l is the
-// whole dot product of nonzero l.  No lane ever has to choose which of two
+// nonzero I ^ l.  Every halving step adds to acc[j] the acc[j + S] of the lane S
+// away, which belongs to the same nonzero; after the last step acc[0] of lane l is
+// the whole dot product of nonzero l.  No lane ever has to choose which of two
 // registers to keep and which to send.  (The lanes of a group then read G
 // different H rows in one instruction: free in LDS, where only banks count.)
 // Otherwise all lanes of a group work on nonzero I in step I and read one
@@ -118,21 +118,24 @@ __device__ __forceinline__ float xor_lane(float v)
     return __int_as_float(from_lane_xor<S>(__float_as_int(v)));
 }
 
-template <int G, bool XORDER, int S = G / 2>
+// XORDER: lane distance 1 first and the largest last, when one register is left:
+// distances 1 and 2 are one v_add with a DPP operand, larger ones cost more.
+template <int G, bool XORDER, int S = XORDER ? 1 : G / 2>
 __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 {
-    if constexpr (S >= 1) {
-        if constexpr (XORDER) {
+    if constexpr (XORDER) {
+        if constexpr (S < G) {
 #pragma unroll
-            for (int j = 0; j < S; ++j) acc[j] += xor_lane<S>(acc[j + S]);
-        } else {
-            const bool upper = (l & S) != 0;
+            for (int j = 0; j < G; j += 2 * S) acc[j] += xor_lane<S>(acc[j + S]);
+            transpose_reduce_step<G, XORDER, S * 2>(acc, l);
+        }
+    } else if constexpr (S >= 1) {
+        const bool upper = (l & S) != 0;
 #pragma unroll
-            for (int j = 0; j < S; ++j) {
-                float keep = upper ? acc[j + S] : acc[j];
-                float send = upper ? acc[j] : acc[j + S];
-                acc[j] = keep + xor_lane<S>(send);
-            }
+        for (int j = 0; j < S; ++j) {
+            float keep = upper ? acc[j + S] : acc[j];
+            float send = upper ? acc[j] : acc[j + S];
+            acc[j] = keep + xor_lane<S>(send);
         }
         transpose_reduce_step<G, XORDER, S / 2>(acc, l);
     }
