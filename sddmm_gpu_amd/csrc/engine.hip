@@ -698,11 +698,12 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1; I.lanes_per_nnz = 8;
 
     if (kernel == SDDMM_KERNEL_HYBRID) {
-        // Rows are split by length into up to three classes:
-        //   long   tile kernel with the default group size: each (row, tile) run is long
-        //          enough to be padded to that group size at little cost
-        //   medium tile kernel with groups of 4 lanes (less padding on short runs)
-        //   short  row gather: a row has so few nonzeros per column tile that padded
+        // Rows are split by length into classes:
+        //   long   tile kernel with the default group size
+        //   medium (only with SDDMM_MED_CLASS=1) tile kernel with groups of 4 lanes: less
+        //          padding on short runs, but twice the W bytes per position through the
+        //          load path, which is what binds it -- measured no faster than "long"
+        //   short  padded gather: a row has so few nonzeros per column tile that padded
         //          runs would mostly be padding
         // How many tiles a row's nonzeros spread over is judged from the column span of
         // panels of consecutive rows, not from n_cols (a banded matrix spans few tiles).
@@ -725,9 +726,9 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         }
         const double tiles = std::max(1.0, span / std::max(1, x));
         const int g_long = pick_tile_variant(kt, 0).G;
-        const bool have_g4 = pick_tile_variant(kt, 4).G != 0 && g_long != 4;
+        const bool have_g4 = env_i64("SDDMM_MED_CLASS", 0) != 0 && pick_tile_variant(kt, 4).G != 0 && g_long != 4;
         int64_t long_min = (int64_t)std::max(2.0 * g_long, 2.0 * g_long * tiles);
-        int64_t short_max = (int64_t)std::max(4.0, (have_g4 ? 2.0 : 1.0 * g_long) * tiles);
+        int64_t short_max = (int64_t)std::max(4.0, (g_long == 8 ? 2.0 : 1.0 * g_long) * tiles);
         long_min = env_i64("SDDMM_LONG_ROW_MIN", long_min);
         short_max = env_i64("SDDMM_SHORT_ROW_MAX", short_max);
         if (!have_g4) long_min = short_max;
@@ -773,9 +774,10 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (!rm.empty()) {
             // (medium rows may use a narrower K slice: wider column tiles, longer runs, more passes)
             int km = (int)env_i64("SDDMM_MED_KSLICE", kt == 128 ? 64 : kt);
-            if (km <= 0 || km > kt || K % km || !pick_tile_variant(km, 4).G) km = kt;
+            int gm = (int)env_i64("SDDMM_MED_G", 4);
+            if (km <= 0 || km > kt || K % km || !pick_tile_variant(km, gm).G) { km = kt; gm = 4; }
             const int32_t xm = km == kt ? x : (int32_t)std::min<int64_t>(kLdsMaxBytes / (km * 4), std::max<int64_t>(n_cols, 1));
-            if (int rc = add_tile(c, rm, xm, y_panel, 4, km, rl.empty() ? &I : &scratch, false, tile_x > 0 && km == kt)) return rc;
+            if (int rc = add_tile(c, rm, xm, y_panel, gm, km, rl.empty() ? &I : &scratch, false, tile_x > 0 && km == kt)) return rc;
         }
         if (!rs.empty()) {
             // short rows: the padded, pipelined kernel reading H from global memory when the

@@ -180,12 +180,12 @@ def test_value_sources_and_host_form(oracle):
         check(d2, out.cpu().numpy(), oracle)
     # the same on a hybrid plan with all three row classes
     import os
-    os.environ.update(SDDMM_LONG_ROW_MIN="150", SDDMM_SHORT_ROW_MAX="15", SDDMM_SPLIT_MIN_NNZ="0")
+    os.environ.update(SDDMM_LONG_ROW_MIN="150", SDDMM_SHORT_ROW_MAX="15", SDDMM_SPLIT_MIN_NNZ="0", SDDMM_MED_CLASS="1")
     try:
         plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, 0, 0,
                                          capi.KERNEL_HYBRID, keep=(rp, ci))
     finally:
-        for k in ("SDDMM_LONG_ROW_MIN", "SDDMM_SHORT_ROW_MAX", "SDDMM_SPLIT_MIN_NNZ"):
+        for k in ("SDDMM_LONG_ROW_MIN", "SDDMM_SHORT_ROW_MAX", "SDDMM_SPLIT_MIN_NNZ", "SDDMM_MED_CLASS"):
             os.environ.pop(k)
     assert sum(plan.info()["class_nnz"]) == d["nnz"]
     plan.set_values(dv.data_ptr())
@@ -232,6 +232,7 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(long_min))
     monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
     monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # split even this small matrix
+    monkeypatch.setenv("SDDMM_MED_CLASS", "1")      # the medium class is off by default
     d = synth.make(3, 0.02, K=128)
     deg = np.diff(d["row_ptr"].numpy())
     out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID)
