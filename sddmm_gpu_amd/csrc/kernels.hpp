@@ -70,9 +70,9 @@ using TileFn = void (*)(const TileArgs);
 // want_g > 0: that group size or nothing; 0: the preferred one for K
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
-// gather: H rows from global memory, 4 waves per workgroup (otherwise H tiles in LDS, 16 waves)
+// gather: H rows from global memory, 4 waves per workgroup (otherwise H tiles in LDS, nwaves = 16 or 12 waves)
 // accumulate: out += instead of out = (K slices after the first)
-TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate);
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
 
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);

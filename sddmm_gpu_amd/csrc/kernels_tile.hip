@@ -394,13 +394,14 @@ TileVariant pick_tile_variant(int K, int want_g)
     return best;
 }
 
-TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate)
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
 {
+#define SDDMM_PICK_NW(g, kpl, vm, nw)                                                                       \
+    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, true> : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
 #define SDDMM_PICK(g, kpl, vm)                                                                              \
     (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, true>                            \
                           : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
-            : (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, 16, false, true>                          \
-                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 16, false, false>))
+            : (nwaves == 12 ? SDDMM_PICK_NW(g, kpl, vm, 12) : SDDMM_PICK_NW(g, kpl, vm, 16)))
 #define SDDMM_CASE(g, kpl)                                                                                  \
     if (v.G == g && v.KPL == kpl)                                                                           \
         return vmode == 0 ? SDDMM_PICK(g, kpl, 0) : vmode == 1 ? SDDMM_PICK(g, kpl, 1) : SDDMM_PICK(g, kpl, 2);
@@ -408,6 +409,7 @@ TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate
     SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
 #undef SDDMM_CASE
 #undef SDDMM_PICK
+#undef SDDMM_PICK_NW
     return nullptr;
 }
 
