@@ -184,14 +184,23 @@ def main():
             sweep[str(K)] = {"gflops": round(r["gflops"], 1), "kernel_ms": round(r["kernel_ms_mean"], 4),
                              "hbm_frac": round(r["frac"], 4)}
         line["gflops_by_K"] = sweep
-    if args.copy_probe:
-        n = 1 << 30
-        a = torch.empty(n // 4, device=dev); b = torch.empty_like(a)
-        a.fill_(1.0)
-        torch.cuda.synchronize()
+    # a plain 1 GiB device-to-device copy next to it: with --copy-probe as the known-size
+    # reference for the HBM counters, always as the bandwidth a streaming kernel reaches here
+    n = 1 << 30
+    a = torch.empty(n // 4, device=dev); b = torch.empty_like(a)
+    a.fill_(1.0)
+    b.copy_(a)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
         b.copy_(a)
-        torch.cuda.synchronize()
+    e1.record()
+    torch.cuda.synchronize()
+    line["roofline"]["measured_copy_gbps"] = round(10 * 2.0 * n / (e0.elapsed_time(e1) * 1e6), 1)
+    if args.copy_probe:
         line["copy_probe_bytes_each_way"] = n
+    del a, b
     if not args.no_cpu:
         set_rank(K0)
         line["cpu_baseline"] = cpu_baseline(d, K0)
