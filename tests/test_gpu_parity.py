@@ -242,3 +242,36 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     if long_min == 200 and short_max == 20:
         assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 4  # 1 + 2 K slices + 1
         assert info["class_rows"][0] == int((deg >= 200).sum())
+
+
+@pytest.mark.parametrize("K,env", [
+    (64, {}), (192, {}), (256, {}), (512, {}),
+    (128, {"SDDMM_TILE_WAVES": "16"}),                      # 16 instead of 12 waves per workgroup
+    (128, {"SDDMM_TILE_ASSIGN": "1"}), (128, {"SDDMM_TILE_ASSIGN": "0"}),   # other work assignments
+    (256, {"SDDMM_TILE_KSLICE": "256"}),                    # one full-K slice: variant G=8, 8 float4 per lane
+    (512, {"SDDMM_TILE_KSLICE": "256"}),                    # two slices of 256
+    (512, {"SDDMM_TILE_KSLICE": "512"}),                    # variant G=16 or 32
+    (128, {"SDDMM_MED_CLASS": "1", "SDDMM_LONG_ROW_MIN": "400"}),   # third class: groups of 4 lanes, K slices of 64
+    (128, {"SDDMM_GATHER_G": "4"}), (256, {"SDDMM_GATHER_PADDED": "0"}),
+])
+def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
+    """The split plan (tile kernel + padded gather) at several ranks and with the
+    planner's alternatives forced through their environment switches."""
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    d = synth.make(3, 0.06, K=K, seed=77)
+    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    check(d, out, oracle)
+    assert sum(info["class_nnz"]) == d["nnz"]
+    assert info["kernel"] == capi.KERNEL_HYBRID and info["class_nnz"][0] > 0 and info["class_nnz"][2] > 0, info
+    # the same plan with the values handed over once must give the same bits
+    dev = torch.device("cuda:0")
+    dd = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], dd["row_ptr"].data_ptr(), dd["col_ind"].data_ptr(),
+                                     K, 0, 0, capi.KERNEL_AUTO)
+    plan.set_values(dd["val"].data_ptr())
+    out2 = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(0, dd["W"].data_ptr(), dd["H"].data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(out2.cpu().numpy(), out)
