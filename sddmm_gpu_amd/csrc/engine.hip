@@ -434,8 +434,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 }
                 // padding repeats the run's last nonzero: the kernel stores every position
                 // without a test, and a repeat stores the same result at the same place
+                const bool flag_padding = gather && env_i64("SDDMM_GATHER_SINK", 1) != 0;
                 for (; d < poff[s + 1]; ++d) {
-                    perm[d] = perm[d - 1];
+                    perm[d] = flag_padding ? (int32_t)((uint32_t)perm[d - 1] | 0x80000000u) : perm[d - 1];
                     scol[d] = scol[d - 1];
                     if (c.vals) sval[d] = sval[d - 1];
                 }
@@ -443,6 +444,26 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             }
         });
         np = np_new;
+        if (gather && env_i64("SDDMM_GATHER_SINK", 1) != 0) {
+            // Gather form: in step I of a batch the 8 groups read the H rows of positions
+            // 64 b + 8 g + I.  A padding position there re-reads its own row's last column: one
+            // more cache line through the load path, which is what binds this kernel.  Point it
+            // at the column another group reads in the same step instead (the same line, merged
+            // by the load path), and flag its index so that the result is dropped.
+            const int64_t nb64 = (np + 63) / 64;
+            parallel_ranges(nb64, 1 << 8, [&](int64_t bb, int64_t be, int) {
+                for (int64_t b = bb; b < be; ++b) {
+                    const int64_t base = b * 64, lim = std::min<int64_t>(np, base + 64);
+                    for (int I = 0; I < G; ++I) {
+                        int32_t common = scol[(size_t)base];  // (a group's first position is never padding)
+                        for (int64_t d = base + I; d < lim; d += G)
+                            if (perm[(size_t)d] >= 0) { common = scol[(size_t)d]; break; }
+                        for (int64_t d = base + I; d < lim; d += G)
+                            if (perm[(size_t)d] < 0) scol[(size_t)d] = common;
+                    }
+                }
+            });
+        }
         if (grid2d) {
             // row-block boundaries: equal shares of the rows' nonzeros
             std::vector<int32_t> cut((size_t)shares + 1, INT32_MAX);
@@ -516,6 +537,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.unit_ptr = d_uptr; a.unit_tile = d_utile;
     L.sval = d_sval; L.perm = d_perm;
     a.n_units = (int32_t)unit_tile.size(); a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
+    if (gather) {
+        float *d_sink = nullptr;
+        if (int rc = c.up(&d_sink, std::vector<float>(256 * 64, 0.f))) return rc;
+        a.sink = d_sink;
+    }
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     if (grid2d) {
         WorkItem *d_items = nullptr;

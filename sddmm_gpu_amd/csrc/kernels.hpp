@@ -54,6 +54,7 @@ struct TileArgs {
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;
+    float *sink;               // gather form: 256 x 64 floats that take the results of flagged padding positions
     const int32_t *unit_ptr;   // [n_units+1] first stream position of each (row panel, column tile) unit
     const int32_t *unit_tile;  // [n_units] the unit's column tile
     int32_t n_units;

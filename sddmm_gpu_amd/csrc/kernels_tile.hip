@@ -278,7 +278,7 @@ void sddmm_tile_kernel(const TileArgs a)
         };
         // ACC (K slices after the first): the previous slices' partial result, requested
         // one batch ahead of its use
-        auto issue_old = [&](Meta &m) { m.old = ACC ? a.out[m.p] : 0.f; };
+        auto issue_old = [&](Meta &m) { m.old = ACC ? a.out[GATHER ? (m.p & 0x7fffffffu) : m.p] : 0.f; };
         // wrow: float4 index of the row's first element in W
         auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
             const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
@@ -290,13 +290,22 @@ void sddmm_tile_kernel(const TileArgs a)
         };
         float pend_v;  // result of the batch before, not yet stored
         uint32_t pend_p;
-        auto flush = [&]() { a.out[pend_p] = pend_v; };
+        // (gather form: a position whose index carries bit 31 is padding that worked on
+        // another row's column; its result goes to a scratch line instead of the output)
+        auto flush = [&]() {
+            if constexpr (GATHER) {
+                float *dst = (int32_t)pend_p < 0 ? a.sink + (((blockIdx.x & 255) << 6) + lane) : a.out + pend_p;
+                *dst = pend_v;
+            } else {
+                a.out[pend_p] = pend_v;
+            }
+        };
         // c[I]: where the H row this lane works on in step I starts (LDS: byte address of
         // this lane's first piece; gather form: float4 index of the row); cn: the same for the next batch, requested here after the last LDS
         // read so that the latency hides behind the reduction
         auto compute = [&](const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
             float v = m.sv;
-            if (VMODE == 1) v = a.val[m.p];
+            if (VMODE == 1) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
             float acc[G];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
