@@ -165,7 +165,7 @@ void sddmm_tile_kernel(const TileArgs a)
     constexpr int NB = GATHER ? 1 : (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL);
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: loop bounds stay in SGPRs
     const int l = lane & (G - 1);
     const int rot = (lane / G) & (NB - 1);
 
