@@ -772,7 +772,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         // staging every H tile must be paid for by the nonzeros that use it
         const int64_t n_tiles_all = (n_cols + x - 1) / x;
         const int64_t stage_rows = std::max<int64_t>(n_tiles_all, c.cus) * x;
-        if (nl + nm < 8 * stage_rows) {
+        if (nl + nm < env_i64("SDDMM_STAGE_FACTOR", 8) * stage_rows) {
             rs.insert(rs.end(), rl.begin(), rl.end()); rs.insert(rs.end(), rm.begin(), rm.end());
             nsh += nl + nm; nl = nm = 0; rl.clear(); rm.clear();
             std::sort(rs.begin(), rs.end());

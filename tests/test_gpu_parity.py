@@ -275,3 +275,40 @@ def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
     plan.execute(0, dd["W"].data_ptr(), dd["H"].data_ptr(), out2.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(out2.cpu().numpy(), out)
+
+
+@pytest.mark.parametrize("seed", list(range(48)))
+def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
+    """Seeded random shapes, densities, ranks, kernels and tile sizes; every second
+    case lets the planner split even a small matrix into its row classes."""
+    rng = np.random.default_rng(1000 + seed)
+    n_rows = int(rng.integers(1, 3000)); n_cols = int(rng.integers(1, 6000))
+    K = int(rng.choice([4, 8, 12, 32, 64, 96, 128, 256, 512]))
+    kernel = str(rng.choice(["auto", "row", "lds", "hybrid", "panel"]))
+    tile_x = int(rng.choice([0, 1, 7, 64, 192, 320, 5000])); tile_y = int(rng.choice([0, 1, 33, 50000]))
+    if seed % 2:
+        monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+        monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")  # tile even where staging the H tiles does not pay
+        monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(int(rng.integers(2, 200))))
+        monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(int(rng.integers(1, 40))))
+    # rows of very unequal length: a few long ones, many short or empty ones
+    deg = np.minimum(n_cols, (rng.pareto(1.2, n_rows) * rng.integers(1, 30)).astype(np.int64))
+    deg[rng.random(n_rows) < 0.2] = 0
+    rows = np.repeat(np.arange(n_rows, dtype=np.int64), deg)
+    cols = rng.integers(0, n_cols, len(rows))
+    key = np.unique(rows * n_cols + cols)
+    if len(key) == 0:
+        key = np.array([0], dtype=np.int64)
+    r = (key // n_cols).astype(np.int32); c = (key % n_cols).astype(np.int32)
+    d = dict(n_rows=n_rows, n_cols=n_cols, nnz=len(r), K=K, row_ind=torch.from_numpy(r), col_ind=torch.from_numpy(c),
+             row_ptr=torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(r, minlength=n_rows))]).astype(np.int32)),
+             val=torch.from_numpy(rng.standard_normal(len(r)).astype(np.float32)),
+             W=torch.from_numpy(rng.standard_normal((n_rows, K)).astype(np.float32)),
+             H=torch.from_numpy(rng.standard_normal((n_cols, K)).astype(np.float32)))
+    out, info = run_gpu(d, tile_x=tile_x, tile_y=tile_y, kernel=KERNELS[kernel])
+    rows_np = d["row_ind"].numpy(); cols_np = d["col_ind"].numpy(); vals = d["val"].numpy()
+    cpu = oracle.sddmm_csr(d["row_ptr"].numpy(), cols_np, vals, d["W"].numpy(), d["H"].numpy())
+    _, absp = oracle.sddmm_f64(rows_np, cols_np, vals, d["W"].numpy(), d["H"].numpy())
+    rep = parity_report(out, cpu, K, absp)
+    assert rep["violations"] == 0, (rep, n_rows, n_cols, K, kernel, tile_x, tile_y, info)
+    assert sum(info["class_nnz"]) == d["nnz"]
