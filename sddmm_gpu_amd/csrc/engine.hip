@@ -528,6 +528,32 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     int32_t *d_perm = nullptr, *d_scol = nullptr, *d_grow = nullptr;
     float *d_sval = nullptr;
     int32_t *d_uptr = nullptr, *d_utile = nullptr;
+    // the compact stream format of narrow K slices (see TileArgs): at K slices of 32 and 64 the
+    // kernel is bound by the bytes it streams (K=32: 0.476 -> 0.411 ms); at 128 it is bound by
+    // VALU issue and the 6 extra instructions per batch cost more than the bytes save.  perm
+    // stays on the device for sddmm_plan_set_values only.
+    const bool compact = !gather && ks / 4 <= 16;
+    if (compact) {
+        const int64_t ng = np / G;
+        std::vector<uint16_t> scol16((size_t)np + kStreamSlack, 0);
+        std::vector<int32_t> pbase((size_t)ng + kStreamSlack, 0);
+        const int32_t row_bytes = ks * 4;
+        parallel_ranges(ng, 1 << 12, [&](int64_t gb, int64_t ge, int) {
+            for (int64_t g = gb; g < ge; ++g) {
+                int cnt = 1;
+                while (cnt < G && perm[(size_t)(g * G + cnt)] != perm[(size_t)(g * G + cnt - 1)]) ++cnt;
+                pbase[(size_t)g] = perm[(size_t)(g * G)];
+                grow[(size_t)g] |= cnt - 1;
+                for (int i = 0; i < G; ++i) scol16[(size_t)(g * G + i)] = (uint16_t)(scol[(size_t)(g * G + i)] / row_bytes);
+            }
+        });
+        uint16_t *d_scol16 = nullptr;
+        int32_t *d_pbase = nullptr;
+        if (int rc = c.up(&d_scol16, scol16)) return rc;
+        if (int rc = c.up(&d_pbase, pbase)) return rc;
+        L.ta.scol16 = d_scol16; L.ta.pbase = d_pbase;
+        std::vector<int32_t>().swap(scol);  // not used by the compact kernels
+    }
     if (int rc = c.up(&d_perm, perm)) return rc;
     if (int rc = c.up(&d_scol, scol)) return rc;
     if (int rc = c.up(&d_grow, grow)) return rc;

@@ -51,6 +51,13 @@ struct TileArgs {
                            // gather form: index of the H row's first float4, column * K/4
     const int32_t *grow;   // per group of G consecutive stream positions: index of the W row's first float4, row * K/4
     const float *sval;     // values in stream order or null
+    // Compact form (LDS tiles of a K slice of at most 64 elements, where the kernel is bound by
+    // the bytes it streams): scol16 replaces scol with the column's index inside the tile,
+    // pbase replaces perm with one word per group of G positions -- the sorted position of
+    // the group's first nonzero; its nonzeros are consecutive there -- and grow carries the
+    // group's number of nonzeros minus one in its low bits (rows are K/4 >= 8 float4 long).
+    const uint16_t *scol16;
+    const int32_t *pbase;
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;

@@ -156,6 +156,8 @@ void sddmm_tile_kernel(const TileArgs a)
     extern __shared__ float4 lds_tile[];
     constexpr int K4 = G * KPL;
     constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
+    constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
+    constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
     // Groups that share one 16-lane LDS access phase read the 16-byte pieces of
     // their rows in different orders (piece j ^ rot instead of j), so that their
     // reads fall into different banks whenever rows are a multiple of 256 bytes
@@ -247,8 +249,9 @@ void sddmm_tile_kernel(const TileArgs a)
         // 64-bit arithmetic, and no load sits behind a branch.
         struct Meta { uint32_t wrow, p; int col; float sv, old; };
         const uint32_t last = (uint32_t)(end - begin - 1);
-        const char *perm_b = reinterpret_cast<const char *>(a.perm + begin);
-        const char *scol_b = reinterpret_cast<const char *>(a.scol + begin);
+        const char *perm_b = reinterpret_cast<const char *>(COMPACT ? a.pbase + begin / G : a.perm + begin);
+        const char *scol_b = COMPACT ? reinterpret_cast<const char *>(a.scol16 + begin)
+                                     : reinterpret_cast<const char *>(a.scol + begin);
         const char *sval_b = reinterpret_cast<const char *>(a.sval + begin);
         const char *grow_b = reinterpret_cast<const char *>(a.grow + begin / G);
         // Steady state: batches are requested in order, two ahead of the one computed,
@@ -258,9 +261,16 @@ void sddmm_tile_kernel(const TileArgs a)
         uint32_t og = (((uint32_t)(b0 << 6) + (uint32_t)lane) / G) << 2;   // grow
         auto issue_meta = [&]() -> Meta {
             Meta m;
-            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + og);
-            m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
-            m.col = *reinterpret_cast<const int *>(scol_b + o4);
+            if constexpr (COMPACT) {
+                const uint32_t g = *reinterpret_cast<const uint32_t *>(grow_b + og);
+                m.wrow = g & ~(uint32_t)(G - 1);
+                m.p = *reinterpret_cast<const uint32_t *>(perm_b + og) + min((uint32_t)l, g & (uint32_t)(G - 1));
+                m.col = (int)*reinterpret_cast<const uint16_t *>(scol_b + (o4 >> 1)) << ROW_SHIFT;
+            } else {
+                m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + og);
+                m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
+                m.col = *reinterpret_cast<const int *>(scol_b + o4);
+            }
             m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
             o4 += 256;
             og += 256 / G;
@@ -270,9 +280,17 @@ void sddmm_tile_kernel(const TileArgs a)
         auto issue_meta_tail = [&](int bi) -> Meta {
             const uint32_t t4 = min((uint32_t)(bi << 6) + (uint32_t)lane, last) << 2;
             Meta m;
-            m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + ((t4 / (4 * G)) << 2));
-            m.p = *reinterpret_cast<const uint32_t *>(perm_b + t4);
-            m.col = *reinterpret_cast<const int *>(scol_b + t4);
+            const uint32_t tg = (t4 / (4 * G)) << 2;
+            if constexpr (COMPACT) {
+                const uint32_t g = *reinterpret_cast<const uint32_t *>(grow_b + tg);
+                m.wrow = g & ~(uint32_t)(G - 1);
+                m.p = *reinterpret_cast<const uint32_t *>(perm_b + tg) + min((t4 >> 2) & (uint32_t)(G - 1), g & (uint32_t)(G - 1));
+                m.col = (int)*reinterpret_cast<const uint16_t *>(scol_b + (t4 >> 1)) << ROW_SHIFT;
+            } else {
+                m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + tg);
+                m.p = *reinterpret_cast<const uint32_t *>(perm_b + t4);
+                m.col = *reinterpret_cast<const int *>(scol_b + t4);
+            }
             m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
             return m;
         };
