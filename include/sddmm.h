@@ -68,6 +68,7 @@ typedef struct sddmm_plan_info {
     int64_t class_nnz[3]; /* nonzeros handled by LDS_TILE, PANEL, ROW_GATHER launches */
     int64_t class_rows[3];
     int64_t padded_positions; /* stream positions of the LDS_TILE launches, padding included */
+    int64_t short_batches;    /* batches of 64 of those positions that run in half the steps */
     double plan_ms;       /* host time spent in the tiling pass + upload */
 } sddmm_plan_info;
 

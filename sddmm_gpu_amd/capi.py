@@ -31,6 +31,7 @@ class PlanInfo(C.Structure):
                 ("k_slice", c_int32), ("n_col_tiles", c_int32), ("n_row_panels", c_int32), ("kernel", c_int32), ("n_launches", c_int32),
                 ("lanes_per_nnz", c_int32), ("lds_bytes", c_int32), ("grid", c_int32), ("block", c_int32),
                 ("n_blocks", c_int64), ("device_bytes", c_int64), ("class_nnz", c_int64 * 3), ("class_rows", c_int64 * 3), ("padded_positions", c_int64),
+                ("short_batches", c_int64),
                 ("plan_ms", c_double)]
 
     def as_dict(self):

@@ -375,6 +375,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         }
         if (grid2d) panel_rows = INT32_MAX;
     }
+    // Short batches (see tile_variant_shorts): the last chunk of a (row, tile) run that holds at
+    // most G/2 nonzeros is kept apart from the full chunks, and eight such chunks make a batch of
+    // their own, which the kernel runs in half the steps.
+    const bool shorts = grid2d && tile_variant_shorts(tv.G, tv.KPL, gather) && env_i64("SDDMM_TILE_SHORT", 1) != 0;
+    std::vector<uint32_t> btype;
     std::vector<WorkItem> items;
     // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
     // inside a panel column tile by column tile, inside a tile rows ascending.  A
@@ -397,10 +402,128 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             return rc;
         n_tiles_all = T.n_tiles;
         const int64_t n_seg = (int64_t)T.active_end.size();
+        // row-block boundaries of the 2-D assignment: equal shares of the rows' nonzeros
+        std::vector<int32_t> cut((size_t)shares + 1, INT32_MAX);
+        cut[0] = 0;
+        if (grid2d) {
+            int64_t acc = 0; int sidx = 1;
+            for (size_t i = 0; i < rows.size() && sidx < shares; ++i) {
+                acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
+                while (sidx < shares && acc >= L.nnz * sidx / shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
+            }
+        }
+        auto seg_range = [&](int sh, int32_t j, int64_t *s0, int64_t *s1) {
+            const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
+            *s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
+            *s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
+        };
+        auto seg_begin = [&](int32_t j, int64_t sg) { return (sg == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[sg - 1]; };
+        // Layout with short batches: an item (row block x tile) is a sequence of whole batches.  Its
+        // runs are cut into chunks of G positions; a run's last chunk with at most G/2 nonzeros is a
+        // short chunk.  Full and short chunks are collected apart, in run order, and every eight of
+        // a kind are written out as the item's next batch; what is left of both at the end makes
+        // the last batch or two, of the full kind.
+        struct ItemLay { int64_t begin, end, batch_base, s0, s1; };
+        std::vector<ItemLay> lay;
+        if (shorts) {
+            if (rb != 0) return fail(SDDMM_ERR_ARG, "plan: short-batch layout with more than one panel");
+            constexpr int kPerBatch = 8;  // groups per batch (G == 8)
+            lay.assign((size_t)T.n_tiles * shares, ItemLay{0, 0, 0, 0, 0});
+            int64_t n_batches = 0;
+            for (int32_t j = 0; j < T.n_tiles; ++j) {
+                if (T.active_ptr[j + 1] > T.active_ptr[j]) {
+                    unit_ptr.push_back((int32_t)np);
+                    unit_tile.push_back(j);
+                }
+                for (int sh = 0; sh < shares; ++sh) {
+                    ItemLay &it = lay[(size_t)j * shares + sh];
+                    seg_range(sh, j, &it.s0, &it.s1);
+                    int64_t nf = 0, ns = 0;
+                    for (int64_t sg = it.s0; sg < it.s1; ++sg) {
+                        const int64_t len = T.active_end[sg] - seg_begin(j, sg), r = len % G;
+                        nf += len / G + (r > G / 2);
+                        ns += (r >= 1 && r <= G / 2);
+                    }
+                    const int64_t n_full_chunks = nf + ns % kPerBatch;
+                    it.begin = np; it.batch_base = n_batches;
+                    it.end = np + (ns / kPerBatch) * 64 + n_full_chunks * G;
+                    n_batches += ns / kPerBatch + (n_full_chunks + kPerBatch - 1) / kPerBatch;
+                    np = it.begin + (it.end - it.begin + 63) / 64 * 64;  // items start on whole batches of their own
+                    if (np >= INT32_MAX - 4096) return fail(SDDMM_ERR_RANGE, "plan: padded stream beyond int32 offsets");
+                }
+            }
+            perm.assign((size_t)np, 0); scol.assign((size_t)np, 0); grow.assign((size_t)(np / G), 0);
+            if (c.vals) sval.assign((size_t)np, 0.f);
+            std::vector<uint8_t> is_short((size_t)n_batches, 0);
+            const int32_t row_bytes = ks * 4;
+            const uint32_t k4 = (uint32_t)(c.K / 4);
+            parallel_ranges((int64_t)lay.size(), 1, [&](int64_t ib, int64_t ie, int) {
+                struct Chunk { int64_t sg, e0; int cnt; };
+                for (int64_t ii = ib; ii < ie; ++ii) {
+                    const ItemLay &it = lay[(size_t)ii];
+                    const int32_t j = (int32_t)(ii / shares);
+                    const int32_t tile_base = (int32_t)((int64_t)j * x);
+                    Chunk fq[kPerBatch], sq[kPerBatch];
+                    int nfq = 0, nsq = 0;
+                    int64_t next = 0;  // the item's next batch
+                    // chunk ch -> the G positions from d0 on; mirrored: positions G/2.. repeat 0..G/2-1
+                    auto put = [&](const Chunk &ch, int64_t d0, bool mirrored) {
+                        const int64_t b = seg_begin(j, ch.sg);
+                        const int span = mirrored ? G / 2 : G;
+                        int64_t d = d0;
+                        for (int i = 0; i < ch.cnt; ++i, ++d) {
+                            const int32_t p = T.tiled_ind[b + ch.e0 + i];
+                            perm[(size_t)d] = p;
+                            scol[(size_t)d] = (c.col_ind[p] - tile_base) * row_bytes;
+                            if (c.vals) sval[(size_t)d] = c.vals[p];
+                        }
+                        for (; d < d0 + span; ++d) {  // padding repeats the chunk's last nonzero
+                            perm[(size_t)d] = perm[(size_t)d - 1]; scol[(size_t)d] = scol[(size_t)d - 1];
+                            if (c.vals) sval[(size_t)d] = sval[(size_t)d - 1];
+                        }
+                        for (; d < d0 + G; ++d) {
+                            perm[(size_t)d] = perm[(size_t)d - span]; scol[(size_t)d] = scol[(size_t)d - span];
+                            if (c.vals) sval[(size_t)d] = sval[(size_t)d - span];
+                        }
+                        grow[(size_t)(d0 / G)] = (int32_t)((uint32_t)T.active_row[ch.sg] * k4);
+                    };
+                    auto emit = [&](const Chunk *q, int n, bool is_s) {
+                        const int64_t d0 = it.begin + next * 64;
+                        for (int k = 0; k < n; ++k) put(q[k], d0 + (int64_t)k * G, is_s);
+                        if (is_s) is_short[(size_t)(it.batch_base + next)] = 1;
+                        ++next;
+                    };
+                    for (int64_t sg = it.s0; sg < it.s1; ++sg) {
+                        const int64_t len = T.active_end[sg] - seg_begin(j, sg);
+                        const int r = (int)(len % G);
+                        for (int64_t e0 = 0; e0 + G <= len; e0 += G) {
+                            fq[nfq++] = {sg, e0, G};
+                            if (nfq == kPerBatch) { emit(fq, nfq, false); nfq = 0; }
+                        }
+                        if (r > G / 2) {
+                            fq[nfq++] = {sg, len - r, r};
+                            if (nfq == kPerBatch) { emit(fq, nfq, false); nfq = 0; }
+                        } else if (r >= 1) {
+                            sq[nsq++] = {sg, len - r, r};
+                            if (nsq == kPerBatch) { emit(sq, nsq, true); nsq = 0; }
+                        }
+                    }
+                    // the rest, as full chunks: at most two batches, the last one possibly partial
+                    for (int k = 0; k < nsq; ++k) {
+                        fq[nfq++] = sq[k];
+                        if (nfq == kPerBatch) { emit(fq, nfq, false); nfq = 0; }
+                    }
+                    if (nfq) emit(fq, nfq, false);
+                }
+            });
+            btype.assign((size_t)((n_batches + 31) / 32) + 8, 0u);
+            for (int64_t b = 0; b < n_batches; ++b)
+                if (is_short[(size_t)b]) { btype[(size_t)(b >> 5)] |= 1u << (b & 31); ++c.P->info.short_batches; }
+        }
         poff.assign((size_t)n_seg + 1, 0);
         seg_tile.assign((size_t)n_seg, 0);
         poff[0] = np;
-        for (int32_t j = 0; j < T.n_tiles; ++j) {
+        for (int32_t j = 0; j < T.n_tiles && !shorts; ++j) {
             if (T.active_ptr[j + 1] > T.active_ptr[j]) {
                 unit_ptr.push_back((int32_t)poff[T.active_ptr[j]]);
                 unit_tile.push_back(j);
@@ -412,11 +535,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 seg_tile[s] = j;
             }
         }
-        const int64_t np_new = poff[n_seg];
+        const int64_t np_new = shorts ? np : poff[n_seg];
         if (np_new >= INT32_MAX - 4096) return fail(SDDMM_ERR_RANGE, "plan: padded stream beyond int32 offsets");
         perm.resize((size_t)np_new); scol.resize((size_t)np_new); grow.resize((size_t)(np_new / G));
         if (c.vals) sval.resize((size_t)np_new);
-        parallel_ranges(n_seg, 1 << 10, [&](int64_t sb, int64_t se, int) {
+        parallel_ranges(shorts ? 0 : n_seg, 1 << 10, [&](int64_t sb, int64_t se, int) {
             for (int64_t s = sb; s < se; ++s) {
                 const int32_t j = seg_tile[s];
                 const int64_t b = (s == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[s - 1];
@@ -465,20 +588,15 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             });
         }
         if (grid2d) {
-            // row-block boundaries: equal shares of the rows' nonzeros
-            std::vector<int32_t> cut((size_t)shares + 1, INT32_MAX);
-            cut[0] = 0;
-            int64_t acc = 0; int sidx = 1;
-            for (size_t i = 0; i < rows.size() && sidx < shares; ++i) {
-                acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
-                while (sidx < shares && acc >= L.nnz * sidx / shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
-            }
             std::vector<int32_t> tiles_ne;
             for (int32_t j = 0; j < T.n_tiles; ++j) if (T.active_ptr[j + 1] > T.active_ptr[j]) tiles_ne.push_back(j);
             auto item_of = [&](int sh, int32_t j) -> WorkItem {
-                const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
-                const int64_t s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
-                const int64_t s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
+                if (shorts) {
+                    const ItemLay &it = lay[(size_t)j * shares + sh];
+                    return {(int32_t)it.begin, (int32_t)it.end, (int32_t)it.batch_base, j};
+                }
+                int64_t s0, s1;
+                seg_range(sh, j, &s0, &s1);
                 return {(int32_t)poff[s0], (int32_t)poff[s1], 0, j};
             };
             // (a work item's positions are addressed by 32-bit byte offsets from its start)
@@ -553,6 +671,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         if (int rc = c.up(&d_pbase, pbase)) return rc;
         L.ta.scol16 = d_scol16; L.ta.pbase = d_pbase;
         std::vector<int32_t>().swap(scol);  // not used by the compact kernels
+    }
+    if (shorts) {
+        uint32_t *d_btype = nullptr;
+        if (int rc = c.up(&d_btype, btype)) return rc;
+        L.ta.btype = d_btype;
     }
     if (int rc = c.up(&d_perm, perm)) return rc;
     if (int rc = c.up(&d_scol, scol)) return rc;

@@ -7,7 +7,7 @@ namespace sddmm {
 
 struct WorkItem {
     int32_t begin, end;   // stream positions
-    int32_t batch_base;   // index of the item's first batch in batch_seg / batch_mask
+    int32_t batch_base;   // index of the item's first batch in batch_seg / batch_mask (tile kernel: in btype)
     int32_t tile;         // column tile staged in LDS (-1: none)
 };
 
@@ -58,6 +58,10 @@ struct TileArgs {
     // group's number of nonzeros minus one in its low bits (rows are K/4 >= 8 float4 long).
     const uint16_t *scol16;
     const int32_t *pbase;
+    // One bit per batch of 64 positions, counted from WorkItem::batch_base inside an item: set for a
+    // "short" batch, whose groups hold at most G/2 nonzeros each, in positions 0 .. G/2-1 and once
+    // more in G/2 .. G-1 (see tile_variant_shorts).  Null: no short batches.
+    const uint32_t *btype;
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;
@@ -75,6 +79,11 @@ struct TileVariant {
     int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL
 };
 using TileFn = void (*)(const TileArgs);
+// Variants that can skip half the steps of a batch marked short in TileArgs::btype.
+constexpr bool tile_variant_shorts(int G, int KPL, bool gather)
+{
+    return !gather && G == 8 && (G * KPL) % 16 == 0 && G * KPL > 16;
+}
 // want_g > 0: that group size or nothing; 0: the preferred one for K
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values

@@ -18,6 +18,12 @@
 // product in register I.  A halving exchange over the G lanes then leaves the
 // whole dot product of nonzero l in lane l, which scales it by S.val and stores
 // it at the nonzero's own position in the output.
+//
+// Short batches (groups of 8 lanes, rows of 128 or 256 elements): the planner
+// collects run ends of at most 4 nonzeros, eight to a batch, and writes each of
+// them twice into its group's 8 positions.  The two halves of the group then
+// work on the same nonzeros, each lane on its own slice, and after 4 of the 8
+// steps one more exchange between the halves completes the dot products.
 #include <hip/hip_runtime.h>
 #include <utility>
 #include "kernels.hpp"
@@ -158,6 +164,12 @@ void sddmm_tile_kernel(const TileArgs a)
     constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
     constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
     constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
+    // SHORTS: a batch may be marked "short" in a.btype: each of its groups then holds at most G/2
+    // nonzeros in its first G/2 positions and the same ones again in the other G/2.  With the
+    // lane-permuted order the upper half of the lanes then works on the same nonzeros as the lower
+    // half, each lane on its own slice, and steps G/2 .. G-1 can be left out: after G/2 steps every
+    // half group holds half of each dot product, and one more exchange adds the two.
+    constexpr bool SHORTS = tile_variant_shorts(G, KPL, GATHER);
     // Groups that share one 16-lane LDS access phase read the 16-byte pieces of
     // their rows in different orders (piece j ^ rot instead of j), so that their
     // reads fall into different banks whenever rows are a multiple of 256 bytes
@@ -216,9 +228,15 @@ void sddmm_tile_kernel(const TileArgs a)
     int cur_tile = -1;
     for (int step = 0; step < n_steps; ++step) {
         int begin, end, tile;
+        int type_base = 0;                     // index of the item's first batch in a.btype
+        // (constant address space: nothing writes the bits while the kernel runs, and only for such
+        // memory does the compiler use scalar loads next to the kernel's own stores)
+        using const_u32_ptr = const __attribute__((address_space(4))) uint32_t *;
+        const_u32_ptr types = nullptr;         // null: no short batches
         if (a.items) {
             const WorkItem wi = a.items[blockIdx.x + step * gridDim.x];
             begin = wi.begin; end = wi.end; tile = wi.tile;
+            if (SHORTS) { type_base = wi.batch_base; types = (const_u32_ptr)(uintptr_t)a.btype; }
         } else {
             begin = max(lo, a.unit_ptr[unit + step]); end = min(hi, a.unit_ptr[unit + step + 1]);
             tile = GATHER ? 0 : a.unit_tile[unit + step];
@@ -238,7 +256,10 @@ void sddmm_tile_kernel(const TileArgs a)
             __syncthreads();
         }
         const int nb = (end - begin + 63) >> 6;
-        const int b0 = (int)((int64_t)nb * wave / NW), b1 = (int)((int64_t)nb * (wave + 1) / NW);
+        // (the division runs on the vector unit; the results are uniform and go back to scalar
+        // registers, so that the batch counter and the batch type bits are scalar work)
+        const int b0 = __builtin_amdgcn_readfirstlane((int)((int64_t)nb * wave / NW));
+        const int b1 = __builtin_amdgcn_readfirstlane((int)((int64_t)nb * (wave + 1) / NW));
         if (b0 >= b1) continue;  // (no barrier below this point inside the tile)
         const int bf = min(b1, (end - begin) >> 6);  // [b0, bf): this wave's batches of 64 whole positions
 
@@ -321,10 +342,12 @@ void sddmm_tile_kernel(const TileArgs a)
         // c[I]: where the H row this lane works on in step I starts (LDS: byte address of
         // this lane's first piece; gather form: float4 index of the row); cn: the same for the next batch, requested here after the last LDS
         // read so that the latency hides behind the reduction
-        auto compute = [&](const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
+        auto compute = [&]<bool SHORT>(std::bool_constant<SHORT>, const float4 (&w)[KPL], const Meta &m, const int (&c)[G],
+                                       int (&cn)[G], int next_col) {
+            constexpr int STEPS = SHORT ? G / 2 : G;
             float v = m.sv;
             if (VMODE == 1) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
-            float acc[G];
+            float acc[STEPS];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
                     float s = 0.f;
@@ -348,15 +371,35 @@ void sddmm_tile_kernel(const TileArgs a)
                     }
                     acc[I] = s;
                 }(), ...);
-            }(std::make_integer_sequence<int, G>{});
+            }(std::make_integer_sequence<int, STEPS>{});
             columns_of_steps<G, XORDER>(next_col, lane_base0, cn);
-            transpose_reduce_step<G, XORDER>(acc, l);
+            if constexpr (SHORT) {
+                transpose_reduce_step<G / 2, XORDER>(acc, l);  // inside each half group
+                acc[0] += xor_lane<G / 2>(acc[0]);             // the other half's slices of the same nonzero
+            } else {
+                transpose_reduce_step<G, XORDER>(acc, l);
+            }
             // The store is left to the start of the next batch (flush): issued here it
             // would sit, unfinished, in front of the loads that batch waits for.  In a
             // whole batch it needs no predicate: a padding position repeats a nonzero of
             // its own group and so writes that nonzero's own result a second time.
             pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
             pend_p = m.p;
+        };
+
+        // the type bits of 32 consecutive batches, held in scalar registers
+        uint32_t type_word = 0;
+        int type_at = -1;
+        auto short_batch = [&](int b) -> bool {
+            if constexpr (!SHORTS) return false;
+            if (!types) return false;
+            const int g = type_base + b;
+            if ((g >> 5) != type_at) { type_at = g >> 5; type_word = types[type_at]; }
+            return (type_word >> (g & 31)) & 1u;
+        };
+        auto run = [&](int b, const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
+            if (short_batch(b)) compute(std::true_type{}, w, m, c, cn, next_col);
+            else compute(std::false_type{}, w, m, c, cn, next_col);
         };
 
         float4 wa[KPL], wb[KPL];
@@ -371,21 +414,21 @@ void sddmm_tile_kernel(const TileArgs a)
             issue_old(m1);
             issue_w(wb, m1.wrow);
             __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
-            compute(wa, m0, ca, cb, m1.col);
+            run(b0, wa, m0, ca, cb, m1.col);
             for (int bi = b0 + 1; bi < bf; bi += 2) {
                 flush();
                 Meta m3 = issue_meta();
                 issue_old(m2);
                 issue_w(wa, m2.wrow);
                 __builtin_amdgcn_sched_barrier(0);
-                compute(wb, m1, cb, ca, m2.col);
+                run(bi, wb, m1, cb, ca, m2.col);
                 if (bi + 1 >= bf) break;
                 flush();
                 Meta m4 = issue_meta();
                 issue_old(m3);
                 issue_w(wb, m3.wrow);
                 __builtin_amdgcn_sched_barrier(0);
-                compute(wa, m2, ca, cb, m3.col);
+                run(bi + 1, wa, m2, ca, cb, m3.col);
                 m1 = m3;
                 m2 = m4;
             }
@@ -398,7 +441,7 @@ void sddmm_tile_kernel(const TileArgs a)
             issue_old(mt);
             issue_w(wa, mt.wrow);
             columns_of_steps<G, XORDER>(mt.col, lane_base0, ca);
-            compute(wa, mt, ca, cb, mt.col);
+            compute(std::false_type{}, wa, mt, ca, cb, mt.col);
             if (begin + (bf << 6) + lane < end) flush();
         }
     }

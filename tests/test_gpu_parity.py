@@ -248,7 +248,7 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     (64, {}), (192, {}), (256, {}), (512, {}),
     (128, {"SDDMM_TILE_WAVES": "16"}),                      # 16 instead of 12 waves per workgroup
     (128, {"SDDMM_TILE_ASSIGN": "1"}), (128, {"SDDMM_TILE_ASSIGN": "0"}),   # other work assignments
-    (256, {"SDDMM_TILE_KSLICE": "256"}),                    # one full-K slice: variant G=8, 8 float4 per lane
+    (256, {"SDDMM_TILE_KSLICE": "256"}),                    # one full-K slice: variant G=16, 4 float4 per lane
     (512, {"SDDMM_TILE_KSLICE": "256"}),                    # two slices of 256
     (512, {"SDDMM_TILE_KSLICE": "512"}),                    # variant G=16 or 32
     (128, {"SDDMM_MED_CLASS": "1", "SDDMM_LONG_ROW_MIN": "400"}),   # third class: groups of 4 lanes, K slices of 64
@@ -275,6 +275,29 @@ def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
     plan.execute(0, dd["W"].data_ptr(), dd["H"].data_ptr(), out2.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(out2.cpu().numpy(), out)
+
+
+@pytest.mark.parametrize("K,env", [(128, {}), (256, {}), (512, {}), (128, {"SDDMM_TILE_WAVES": "16"})])
+def test_short_batches(oracle, monkeypatch, K, env):
+    """Run ends with at most four nonzeros are collected, eight to a batch, into
+    batches that the tile kernel runs in half the steps (both halves of a group of
+    eight lanes then hold the same nonzeros).  The plan must report such batches, the
+    results must stay within the tolerance of the oracle, two executes must give the
+    same bits (the duplicate positions store the same value to the same place), and
+    with the switch off there are none."""
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    d = synth.make(3, 0.06, K=K, seed=5)
+    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    check(d, out, oracle)
+    assert info["short_batches"] > 0 and info["short_batches"] * 64 < info["padded_positions"], info
+    out_again, _ = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    assert np.array_equal(out, out_again)
+    monkeypatch.setenv("SDDMM_TILE_SHORT", "0")
+    out_off, info_off = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    check(d, out_off, oracle)
+    assert info_off["short_batches"] == 0 and info_off["padded_positions"] <= info["padded_positions"]
 
 
 @pytest.mark.parametrize("seed", list(range(48)))
