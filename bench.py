@@ -102,6 +102,8 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0)
     ap.add_argument("--K", type=int, default=None)
     ap.add_argument("--kernel", default="auto", choices=["auto", "row", "lds", "panel", "hybrid"])
+    ap.add_argument("--epilogue", default="scale", choices=["scale", "residual"],
+                    help="scale: out = val*dot (the reference's form, the default); residual: out = val - dot, fused")
     ap.add_argument("--tile-x", type=int, default=0)
     ap.add_argument("--tile-y", type=int, default=0)
     ap.add_argument("--no-sweep", action="store_true", help="skip the K = 32, 128, 256, 512 report")
@@ -147,7 +149,10 @@ def main():
         plan.set_values(d["val"].data_ptr(), torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         vp, wp, hp, op = 0, d["W"].data_ptr(), d["H"].data_ptr(), out.data_ptr()
-        wall, mean_ev, med_ev = time_steps(lambda s: plan.execute(vp, wp, hp, op, s), args.steps, args.warmup, torch,
+        epi = capi.EPILOGUE_RESIDUAL if args.epilogue == "residual" else capi.EPILOGUE_SCALE
+        run = (lambda s: plan.execute(vp, wp, hp, op, s)) if args.epilogue == "scale" else \
+              (lambda s: plan.execute_epilogue(vp, wp, hp, op, epi, s))
+        wall, mean_ev, med_ev = time_steps(run, args.steps, args.warmup, torch,
                                            args.spinup_ms)
         prof = plan.execute_profiled(vp, wp, hp, op, torch.cuda.current_stream().cuda_stream)
         flops = 2.0 * d["nnz"] * K
@@ -178,7 +183,7 @@ def main():
                    "kernel": KERNEL_NAMES[info["kernel"]], "tile_size_x": info["tile_size_x"],
                    "tile_size_y": info["tile_size_y"], "k_slice": info["k_slice"],
                    "kernel_launches_per_step": info["n_launches"], "plan_ms": round(info["plan_ms"], 1),
-                   "spinup_ms": args.spinup_ms},
+                   "spinup_ms": args.spinup_ms, "epilogue": args.epilogue},
         "roofline": {"bound": "hbm", "achieved": round(main_res["alg_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(main_res["frac"], 4),
                      "traffic": MEASURED_TRAFFIC.get((args.config, args.scale, K0, args.kernel, args.tile_x, args.tile_y)),

@@ -203,6 +203,18 @@ void sddmm_plan_destroy(sddmm_plan *plan);
 int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
                   float *d_out, void *stream);
 
+/* sddmm_execute with the per-nonzero epilogue chosen by the caller, fused into
+ * the kernels' store (no second pass over out):
+ *   SDDMM_EPILOGUE_SCALE     out[p] = val[p] * dot    (= sddmm_execute; sddmm.cu:173)
+ *   SDDMM_EPILOGUE_RESIDUAL  out[p] = val[p] - dot    (needs values: d_val or plan-owned)
+ * The residual is the error term of the matrix-factorisation updates (ALS,
+ * SGD) that the reference names as the use of SDDMM (README.md:1); the
+ * reference itself computes the scaled form only.                           */
+#define SDDMM_EPILOGUE_SCALE 0
+#define SDDMM_EPILOGUE_RESIDUAL 1
+int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                           float *d_out, int32_t epilogue, void *stream);
+
 /* The same execution with an event after every launch-list entry: fills one
  * profile per entry (sddmm_plan_launch_count of them) with its wall time on
  * the device, then returns (synchronises on the last event).  No counterpart

@@ -77,6 +77,17 @@ def sddmm_csr(row_ptr, col_ind, val, W, H, nthreads=0):
     return out
 
 
+def sddmm_residual_csr(row_ptr, col_ind, val, W, H, nthreads=0):
+    """p[ind] = val[ind] - (sum_t W[r,t]*H[c,t]), sequential fp32 sum."""
+    row_ptr, col_ind, val, W, H = _i32(row_ptr), _i32(col_ind), _f32(val), _f32(W), _f32(H)
+    n_rows = len(row_ptr) - 1
+    k = W.shape[1]
+    out = np.empty(len(col_ind), np.float32)
+    lib().oracle_sddmm_residual_csr(c_int64(n_rows), _p(row_ptr), _p(col_ind), _p(val), c_int32(k), _p(W), _p(H), _p(out),
+                                    c_int(nthreads))
+    return out
+
+
 def sddmm_coo(row_ind, col_ind, val, W, H, nthreads=0, apply_val=True, timed=False):
     row_ind, col_ind, val, W, H = _i32(row_ind), _i32(col_ind), _f32(val), _f32(W), _f32(H)
     k = W.shape[1]

@@ -13,6 +13,9 @@
  *   oracle_sddmm_csr / _coo  closed forms (W=H=1, K=1, one-hot H, dense
  *                            S vs a library GEMM, power-of-two scaling),
  *                            fp64 brute force on tiny inputs
+ *   oracle_sddmm_residual_csr  the same loop with the last operation
+ *                            changed: equals val - oracle_sddmm_csr(val = 1)
+ *                            bit for bit (tested), closed form W=H=1
  *   oracle_make_csr,
  *   oracle_rewrite_1d        known answer obtained from the reference's own
  *                            util.h, and oracle/_ref (that header compiled
@@ -55,6 +58,32 @@ void oracle_sddmm_csr(int64_t n_rows, const int32_t *row_ptr,
                 sm = sm + prod;
             }
             p[ind] = sm * val[ind];
+        }
+    }
+}
+
+/* The residual form val - dot over CSR: the loop of sddmm.cu:153-177 with the
+ * last operation changed from sm * val[ind] to val[ind] - sm (the error term
+ * of the matrix-factorisation updates that README.md:1 names as the use of
+ * SDDMM; the reference has no such function).                              */
+void oracle_sddmm_residual_csr(int64_t n_rows, const int32_t *row_ptr,
+                               const int32_t *col_ind, const float *val, int32_t k,
+                               const float *W, const float *H, float *p, int nthreads)
+{
+#ifdef _OPENMP
+    if (nthreads > 0) omp_set_num_threads(nthreads);
+#endif
+    #pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        for (int64_t ind = row_ptr[r]; ind < row_ptr[r + 1]; ++ind) {
+            const float *w = W + (int64_t)r * k;
+            const float *h = H + (int64_t)col_ind[ind] * k;
+            float sm = 0.0f;
+            for (int32_t t = 0; t < k; ++t) {
+                float prod = w[t] * h[t];
+                sm = sm + prod;
+            }
+            p[ind] = val[ind] - sm;
         }
     }
 }

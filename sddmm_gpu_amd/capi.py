@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libsddmm_hip.so")
 
 OK, ERR_ARG, ERR_IO, ERR_FORMAT, ERR_RANGE, ERR_UNSORTED, ERR_HIP, ERR_NOMEM = range(8)
 KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL, KERNEL_HYBRID = 0, 1, 2, 3, 4
+EPILOGUE_SCALE, EPILOGUE_RESIDUAL = 0, 1
 
 
 class SddmmError(RuntimeError):
@@ -77,6 +78,7 @@ SIGNATURES = {
     "sddmm_plan_get_info": (c_int, [c_void_p, POINTER(PlanInfo)]),
     "sddmm_plan_destroy": (None, [c_void_p]),
     "sddmm_execute": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sddmm_execute_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
     "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
     "sddmm_execute_profiled": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(LaunchProfile), c_int32]),
     "sddmm_gpu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_float)]),
@@ -250,6 +252,10 @@ class Plan:
     def execute(self, d_val, d_W, d_H, d_out, stream=0):
         check(lib().sddmm_execute(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
                                   c_void_p(stream or None)))
+
+    def execute_epilogue(self, d_val, d_W, d_H, d_out, epilogue, stream=0):
+        check(lib().sddmm_execute_epilogue(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
+                                           c_int32(epilogue), c_void_p(stream or None)))
 
     def execute_profiled(self, d_val, d_W, d_H, d_out, stream=0):
         n = c_int32()

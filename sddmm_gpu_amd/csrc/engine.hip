@@ -38,7 +38,8 @@ struct Launch {
     KernelFn fn = nullptr;   // stream kernels
     PanelFn pfn = nullptr;   // panel kernel
     TileFn tfn = nullptr;        // tile kernel (values in stream order, first K slice); null: not a tile launch
-    TileFn tfns[3][2] = {};      // [values in stream order / in sorted order / none][first K slice / later slices]
+    TileFn tfns[5][2] = {};      // [values in stream order / in sorted order / none / residual epilogue with values
+                                 //  in stream order / in sorted order][first K slice / later slices]
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
@@ -333,7 +334,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     if (!gather && nwaves != 12) nwaves = 16;
     L.tfn = tv.G ? tile_kernel(tv, 0, gather, false, nwaves) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
-    for (int vm = 0; vm < 3; ++vm)
+    for (int vm = 0; vm < 5; ++vm)
         for (int ac = 0; ac < 2; ++ac) L.tfns[vm][ac] = tile_kernel(tv, vm, gather, ac != 0, nwaves);
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
@@ -702,7 +703,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
     L.k_slice = ks;
     if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
-    for (int vm = 0; vm < 3; ++vm)
+    for (int vm = 0; vm < 5; ++vm)
         for (int ac = 0; ac < 2; ++ac)
             HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
     if (I) {
@@ -1081,14 +1082,16 @@ static int check_execute_args(const sddmm_plan *plan, const float *d_W, const fl
 
 // Issues the kernels of one launch-list entry (one per K slice) on `stream`.
 static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d_val, const float *d_W,
-                         const float *d_H, float *d_out, hipStream_t stream)
+                         const float *d_H, float *d_out, hipStream_t stream, int epilogue = SDDMM_EPILOGUE_SCALE)
 {
+    const int residual = epilogue == SDDMM_EPILOGUE_RESIDUAL;
     const sddmm_plan_info &I = plan->info;
     const float *val = d_val ? d_val : plan->d_val;
     if (L.kind == SDDMM_KERNEL_PANEL) {
         PanelArgs pa = L.pa;
         pa.row_ptr = plan->d_row_ptr; pa.col_ind = plan->d_col;
         pa.val = val; pa.W = d_W; pa.H = d_H; pa.out = d_out;
+        pa.residual = residual;
         for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
             pa.k_off = k_off;
             pa.accumulate = k_off > 0;
@@ -1099,7 +1102,7 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.val = val;
         ta.sval = d_val ? nullptr : L.sval;
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
-        const int vm = ta.sval ? 0 : (val ? 1 : 2);
+        const int vm = residual ? (ta.sval ? 3 : 4) : ta.sval ? 0 : (val ? 1 : 2);
         for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
             ta.k_off = k_off;
             hipLaunchKernelGGL(L.tfns[vm][k_off > 0], dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
@@ -1110,6 +1113,7 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         a.val = val;
         a.sval = d_val ? nullptr : L.sval;
         a.W = d_W; a.H = d_H; a.out = d_out;
+        a.residual = residual;
         hipLaunchKernelGGL(L.fn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, a);
     }
 }
@@ -1120,6 +1124,20 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
     if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute")) return rc;
     if (plan->info.nnz == 0) return SDDMM_OK;
     for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream);
+    HIP_TRY(hipGetLastError());
+    return SDDMM_OK;
+}
+
+int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H, float *d_out,
+                           int32_t epilogue, void *stream)
+{
+    if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute_epilogue")) return rc;
+    if (epilogue != SDDMM_EPILOGUE_SCALE && epilogue != SDDMM_EPILOGUE_RESIDUAL)
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_epilogue: unknown epilogue %d", (int)epilogue);
+    if (epilogue == SDDMM_EPILOGUE_RESIDUAL && !d_val && !plan->d_val && plan->info.nnz > 0)
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_epilogue: the residual val - dot needs values (d_val or plan-owned)");
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream, epilogue);
     HIP_TRY(hipGetLastError());
     return SDDMM_OK;
 }

@@ -30,6 +30,7 @@ struct KArgs {
     int32_t tile_x;
     int32_t n_cols;
     int32_t generic_perm;
+    int32_t residual;          // 0: out = val * dot;  1: out = val - dot
 };
 
 constexpr int kRowGatherBlock = 256;   // 4 waves
@@ -107,6 +108,7 @@ struct PanelArgs {
     int32_t K;                // row length of W and H
     int32_t k_off;            // first K element covered by this pass
     int32_t accumulate;       // add to out instead of overwriting it
+    int32_t residual;         // 0: out = val * dot;  1: out = val - dot (later K slices: out -= dot)
 };
 struct PanelVariant {
     int KPL, S, NWAVES;       // float4 per lane (K slice = 32*KPL), row slots per 8-lane group, waves per workgroup

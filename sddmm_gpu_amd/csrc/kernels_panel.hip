@@ -142,7 +142,7 @@ void sddmm_panel_kernel(const PanelArgs a)
                         const int cnt = __popcll((bal >> (gid * 8)) & 0xffull);
                         if (in) {
                             const int idx = cur[s] + l;
-                            float res = sum * qval[s];
+                            float res = a.residual ? (a.accumulate ? -sum : qval[s] - sum) : sum * qval[s];
                             if (a.accumulate) res += a.out[idx];
                             a.out[idx] = res;
                         }

@@ -220,7 +220,7 @@ void sddmm_stream_kernel(const KArgs a)
                 }(std::make_integer_sequence<int, G>{});
             }
             const float sum = transpose_reduce<G>(acc, l);
-            if (cur.row >= 0) a.out[cur.p] = sum * cur.v;
+            if (cur.row >= 0) a.out[cur.p] = a.residual ? cur.v - sum : sum * cur.v;
         }
     }
 }
@@ -269,7 +269,7 @@ void sddmm_generic_kernel(const KArgs a)
             acc[i] = s;
         }
         const float sum = transpose_reduce<G>(acc, l);
-        if (valid) a.out[p] = sum * v;
+        if (valid) a.out[p] = a.residual ? v - sum : sum * v;
     }
 }
 

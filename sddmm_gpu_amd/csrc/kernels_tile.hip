@@ -148,7 +148,9 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 }
 
 // VMODE: where S.val comes from -- 0: a.sval (stream order), 1: a.val (sorted
-// order, read through the position), 2: nowhere (no scaling).
+// order, read through the position), 2: nowhere (no scaling); 3 and 4: as 0 and 1
+// with the residual epilogue, out = val - dot (K slices after the first: out -= dot,
+// no value needed).
 //
 // The loop is software-pipelined by hand and free of branches around loads, so
 // that every wait is for exactly the data needed: while batch b is computed,
@@ -161,6 +163,9 @@ void sddmm_tile_kernel(const TileArgs a)
 {
     extern __shared__ float4 lds_tile[];
     constexpr int K4 = G * KPL;
+    constexpr bool RESIDUAL = VMODE >= 3;
+    constexpr bool STREAM_VAL = VMODE == 0 || (VMODE == 3 && !ACC);  // values read in stream order
+    constexpr bool SORTED_VAL = VMODE == 1 || (VMODE == 4 && !ACC);  // values read through the position
     constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
     constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
     constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
@@ -292,7 +297,7 @@ void sddmm_tile_kernel(const TileArgs a)
                 m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
                 m.col = *reinterpret_cast<const int *>(scol_b + o4);
             }
-            m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
+            m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
             o4 += 256;
             og += 256 / G;
             return m;
@@ -312,7 +317,7 @@ void sddmm_tile_kernel(const TileArgs a)
                 m.p = *reinterpret_cast<const uint32_t *>(perm_b + t4);
                 m.col = *reinterpret_cast<const int *>(scol_b + t4);
             }
-            m.sv = (VMODE == 0) ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
+            m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
             return m;
         };
         // ACC (K slices after the first): the previous slices' partial result, requested
@@ -346,7 +351,7 @@ void sddmm_tile_kernel(const TileArgs a)
                                        int (&cn)[G], int next_col) {
             constexpr int STEPS = SHORT ? G / 2 : G;
             float v = m.sv;
-            if (VMODE == 1) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
+            if (SORTED_VAL) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
             float acc[STEPS];
             [&]<int... I>(std::integer_sequence<int, I...>) {
                 ((void)[&] {
@@ -383,7 +388,8 @@ void sddmm_tile_kernel(const TileArgs a)
             // would sit, unfinished, in front of the loads that batch waits for.  In a
             // whole batch it needs no predicate: a padding position repeats a nonzero of
             // its own group and so writes that nonzero's own result a second time.
-            pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
+            if constexpr (RESIDUAL) pend_v = ACC ? m.old - acc[0] : v - acc[0];
+            else pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
             pend_p = m.p;
         };
 
@@ -467,14 +473,16 @@ TileVariant pick_tile_variant(int K, int want_g)
 TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
 {
 #define SDDMM_PICK_NW(g, kpl, vm, nw)                                                                       \
-    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, true> : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
+    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, false, true>                    \
+                : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
 #define SDDMM_PICK(g, kpl, vm)                                                                              \
-    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, true>                            \
+    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), 4, true, true>            \
                           : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
             : (nwaves == 12 ? SDDMM_PICK_NW(g, kpl, vm, 12) : SDDMM_PICK_NW(g, kpl, vm, 16)))
 #define SDDMM_CASE(g, kpl)                                                                                  \
     if (v.G == g && v.KPL == kpl)                                                                           \
-        return vmode == 0 ? SDDMM_PICK(g, kpl, 0) : vmode == 1 ? SDDMM_PICK(g, kpl, 1) : SDDMM_PICK(g, kpl, 2);
+        return vmode == 0 ? SDDMM_PICK(g, kpl, 0) : vmode == 1 ? SDDMM_PICK(g, kpl, 1) : vmode == 2 ? SDDMM_PICK(g, kpl, 2)      \
+             : vmode == 3 ? SDDMM_PICK(g, kpl, 3) : SDDMM_PICK(g, kpl, 4);
     SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
     SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
 #undef SDDMM_CASE

@@ -198,6 +198,63 @@ def test_value_sources_and_host_form(oracle):
     assert ms > 0
 
 
+def residual_ok(out, d, oracle, K):
+    """|gpu - cpu| of val - dot within the tolerance of the dot product (the error is
+    the dot product's) plus one rounding of the subtraction."""
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    W = d["W"].numpy(); H = d["H"].numpy()
+    cpu = oracle.sddmm_residual_csr(d["row_ptr"].numpy(), cols, vals, W, H)
+    dot = oracle.sddmm_csr(d["row_ptr"].numpy(), cols, np.ones_like(vals), W, H)
+    _, absp = oracle.sddmm_f64(rows, cols, np.ones_like(vals), W, H)
+    tol = 1e-5 * np.sqrt(K)
+    bound = tol * np.maximum(np.abs(dot), absp / 100.0) + 2.0 ** -23 * np.abs(cpu)
+    assert out.shape == cpu.shape and np.all(np.isfinite(out))
+    bad = np.abs(out.astype(np.float64) - cpu) > bound
+    assert not bad.any(), (int(bad.sum()), float(np.abs(out - cpu).max()))
+
+
+@pytest.mark.parametrize("kernel,K", [("row", 32), ("row", 100), ("row", 30), ("lds", 64), ("lds", 100), ("panel", 128),
+                                      ("panel", 512), ("auto", 32), ("auto", 64), ("auto", 128), ("auto", 256), ("auto", 512)])
+def test_residual_epilogue(oracle, monkeypatch, kernel, K):
+    """out = val - dot fused into every kernel family's store, with the values owned
+    by the plan (stream order) and passed at execute (sorted order), in one K slice
+    and in several; the scaled form through the same entry point gives sddmm_execute's bits."""
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+    d = synth.make(3, 0.05, K=K, seed=21)
+    dev = torch.device("cuda:0")
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    plan = S.plan(K, 0, 0, KERNELS[kernel])
+    W = d["W"].to(dev); H = d["H"].to(dev); dv = d["val"].to(dev)
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
+    torch.cuda.synchronize()
+    residual_ok(out.cpu().numpy(), d, oracle, K)
+    out2 = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute_epilogue(dv.data_ptr(), W.data_ptr(), H.data_ptr(), out2.data_ptr(), capi.EPILOGUE_RESIDUAL)
+    torch.cuda.synchronize()
+    residual_ok(out2.cpu().numpy(), d, oracle, K)
+    a = torch.empty(d["nnz"], device=dev); b = torch.empty(d["nnz"], device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), a.data_ptr())
+    plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), b.data_ptr(), capi.EPILOGUE_SCALE)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_residual_epilogue_needs_values():
+    d = synth.make(1, 0.25)
+    dev = torch.device("cuda:0")
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), d["K"], 0, 0,
+                                     capi.KERNEL_AUTO, keep=(rp, ci))
+    W = d["W"].to(dev); H = d["H"].to(dev); out = torch.empty(d["nnz"], device=dev)
+    with pytest.raises(capi.SddmmError) as e:
+        plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
+    assert e.value.code == capi.ERR_ARG
+    with pytest.raises(capi.SddmmError) as e:
+        plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), 7)
+    assert e.value.code == capi.ERR_ARG
+
+
 def test_device_plan_rejects_bad_csr():
     dev = torch.device("cuda:0")
     rp = torch.tensor([0, 2, 3], dtype=torch.int32, device=dev)

@@ -113,6 +113,26 @@ def test_power_of_two_scaling_and_shipping_form(oracle):
     assert np.array_equal(oracle.sddmm_coo(rows, cols, val, W, H, nthreads=3), base)
 
 
+def test_residual_form_is_the_same_loop_with_another_last_operation(oracle):
+    """val - dot: bit for bit val minus the (pinned) scaled form run with val = 1;
+    closed form W = H = 1 -> val - K; fp64 brute force on a tiny case."""
+    rng = np.random.default_rng(11)
+    n_rows, n_cols, K = 37, 53, 24
+    rows, cols = rand_sorted_coo(rng, n_rows, n_cols, 400)
+    rp = row_ptr_of(rows, n_rows)
+    val = rng.standard_normal(len(rows)).astype(np.float32)
+    W = rng.standard_normal((n_rows, K)).astype(np.float32)
+    H = rng.standard_normal((n_cols, K)).astype(np.float32)
+    res = oracle.sddmm_residual_csr(rp, cols, val, W, H)
+    dot = oracle.sddmm_csr(rp, cols, np.ones_like(val), W, H)
+    assert np.array_equal(res, val - dot)
+    f64 = val.astype(np.float64) - np.einsum("ij,ij->i", W[rows].astype(np.float64), H[cols].astype(np.float64))
+    assert np.abs(res - f64).max() <= 1e-5 * np.sqrt(K) * np.abs(W[rows] * H[cols]).sum(1).max()
+    ones = oracle.sddmm_residual_csr(rp, cols, val, np.ones_like(W), np.ones_like(H))
+    assert np.array_equal(ones, val - np.float32(K))
+    assert np.array_equal(oracle.sddmm_residual_csr(rp, cols, val, W, H, nthreads=1), res)
+
+
 def test_permuting_nonzeros_permutes_outputs(oracle):
     rng = np.random.default_rng(6)
     rows, cols = rand_sorted_coo(rng, 40, 50, 500)
