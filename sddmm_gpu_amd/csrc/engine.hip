@@ -380,6 +380,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // most G/2 nonzeros is kept apart from the full chunks, and eight such chunks make a batch of
     // their own, which the kernel runs in half the steps.
     const bool shorts = grid2d && tile_variant_shorts(tv.G, tv.KPL, gather) && env_i64("SDDMM_TILE_SHORT", 1) != 0;
+    // gather form: padding positions are flagged and their results go to a scratch line
+    const bool flag_padding = gather && env_i64("SDDMM_GATHER_SINK", 1) != 0;
+    const bool deal_tiles = env_i64("SDDMM_TILE_DEAL", 1) != 0;
     std::vector<uint32_t> btype;
     std::vector<WorkItem> items;
     // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
@@ -558,7 +561,6 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 }
                 // padding repeats the run's last nonzero: the kernel stores every position
                 // without a test, and a repeat stores the same result at the same place
-                const bool flag_padding = gather && env_i64("SDDMM_GATHER_SINK", 1) != 0;
                 for (; d < poff[s + 1]; ++d) {
                     perm[d] = flag_padding ? (int32_t)((uint32_t)perm[d - 1] | 0x80000000u) : perm[d - 1];
                     scol[d] = scol[d - 1];
@@ -568,7 +570,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             }
         });
         np = np_new;
-        if (gather && env_i64("SDDMM_GATHER_SINK", 1) != 0) {
+        if (flag_padding) {
             // Gather form: in step I of a batch the 8 groups read the H rows of positions
             // 64 b + 8 g + I.  A padding position there re-reads its own row's last column: one
             // more cache line through the load path, which is what binds this kernel.  Point it
@@ -615,7 +617,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                             const WorkItem it = item_of(die, j);
                             ld[(size_t)j] = {-(int64_t)(it.end - it.begin), j};
                         }
-                        if (env_i64("SDDMM_TILE_DEAL", 1) != 0) std::sort(ld.begin(), ld.end());
+                        if (deal_tiles) std::sort(ld.begin(), ld.end());
                         for (int step = 0; step < xcd_steps; ++step)
                             for (int slot = 0; slot < per_die; ++slot)
                                 deal[(size_t)die * nt + (size_t)step * per_die + slot] =
