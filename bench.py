@@ -24,7 +24,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
 # the default workload (see profiles/*hbm_traffic*.txt for the runs and the
 # copy-kernel scale factors); None where no such measurement exists.
-MEASURED_TRAFFIC = {(3, 1.0, 128, "auto", 0, 0): 3.13e9}
+MEASURED_TRAFFIC = {(3, 1.0, 128, "auto", 0, 0): 3.14e9}
 
 
 def alg_bytes(nnz, n_rows, K, rows_touched, cols_touched):
