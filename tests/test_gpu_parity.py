@@ -116,6 +116,48 @@ def test_edge_shapes(oracle):
             check(d, out, oracle)
 
 
+def _dict_of(n, m, r, c, K, rng):
+    r = np.asarray(r, np.int32); c = np.asarray(c, np.int32)
+    order = np.lexsort((c, r)); r = r[order]; c = c[order]
+    return dict(n_rows=n, n_cols=m, nnz=len(r), K=K, row_ind=torch.from_numpy(r), col_ind=torch.from_numpy(c),
+                row_ptr=torch.from_numpy(np.concatenate([[0], np.cumsum(np.bincount(r, minlength=n))]).astype(np.int32)),
+                val=torch.from_numpy(rng.standard_normal(len(r)).astype(np.float32)),
+                W=torch.from_numpy(rng.standard_normal((n, K)).astype(np.float32)),
+                H=torch.from_numpy(rng.standard_normal((m, K)).astype(np.float32)))
+
+
+@pytest.mark.parametrize("forced", [False, True])
+def test_extreme_shapes_through_the_planner(oracle, monkeypatch, forced):
+    """Degenerate shapes through AUTO and HYBRID, once with the planner's own choices
+    and once with its size thresholds removed, so that the tiled and split plans (and
+    their short batches) are built for inputs they would normally never see."""
+    if forced:
+        monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+        monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")
+    rng = np.random.default_rng(123)
+    wide = np.unique(rng.integers(0, 150000, 60000))
+    cases = [
+        ("one_by_one", 1, 1, [0], [0], 128),
+        ("one_long_row", 1, 150000, np.zeros(len(wide)), wide, 128),
+        ("one_long_col", 150000, 1, wide, np.zeros(len(wide)), 128),
+        ("one_row_of_three", 3, 700, [1, 1, 1], [0, 350, 699], 128),
+        ("dense_block", 96, 640, np.repeat(np.arange(96), 640), np.tile(np.arange(640), 96), 128),
+        ("dense_block_k256", 64, 300, np.repeat(np.arange(64), 300), np.tile(np.arange(300), 64), 256),
+        ("runs_of_1_to_9", 45, 600, np.repeat(np.arange(45), np.arange(45) % 9 + 1),
+         np.concatenate([np.arange(k % 9 + 1) * 7 + k for k in range(45)]), 128),
+        ("rank_4", 500, 400, *np.divmod(np.unique(rng.integers(0, 500 * 400, 9000)), 400), 4),
+        ("rank_8", 500, 400, *np.divmod(np.unique(rng.integers(0, 500 * 400, 9000)), 400), 8),
+        ("rank_1024", 120, 90, *np.divmod(np.unique(rng.integers(0, 120 * 90, 3000)), 90), 1024),
+        ("rank_2048", 60, 50, *np.divmod(np.unique(rng.integers(0, 60 * 50, 900)), 50), 2048),
+    ]
+    for name, n, m, r, c, K in cases:
+        d = _dict_of(n, m, r, c, K, rng)
+        for kernel in ("auto", "hybrid"):
+            out, info = run_gpu(d, kernel=KERNELS[kernel])
+            rep = check(d, out, oracle)
+            assert sum(info["class_nnz"]) == d["nnz"], (name, kernel, info)
+
+
 def test_empty_matrix_and_empty_rows(oracle):
     S = capi.Coo.from_arrays(10, 10, [], [])
     plan = S.plan(32)
