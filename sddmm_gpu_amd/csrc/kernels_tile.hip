@@ -1,459 +1,6 @@
-// Tile kernel of the SDDMM engine for gfx950 (MI355X): column tiles of H in
-// LDS, nonzeros streamed in tile order with every (row, tile) run padded to a
-// multiple of G positions.
-//
-// The stream lists S tile by tile (tiles of tile_x columns), rows ascending
-// inside a tile; scol holds, instead of the column, the byte offset of the
-// column's H row inside the LDS tile.  Each run of one row inside one tile is
-// padded to a multiple of G positions (the padding repeats the run's last
-// nonzero), so a group of G lanes always works on ONE row: there is no
-// per-nonzero row test in the inner loop.  A batch is 64 consecutive stream
-// positions, one per lane.  While batch b is computed, the index data of batch
-// b+2 (output position, LDS offset, value, W row) and the W row slices of
-// batch b+1 are in flight, and the result of batch b-1 is being stored.  Lane l
-// of a group holds slice l of the row's W elements; in step I it reads the same
-// slice of the H row of one of the group's nonzeros from LDS (in 16-byte pieces;
-// the groups sharing one 16-lane LDS phase visit the pieces in different orders,
-// so their reads fall into different banks) and accumulates the partial dot
-// product in register I.  A halving exchange over the G lanes then leaves the
-// whole dot product of nonzero l in lane l, which scales it by S.val and stores
-// it at the nonzero's own position in the output.
-//
-// Short batches (groups of 8 lanes, rows of 128 or 256 elements): the planner
-// collects run ends of at most 4 nonzeros, eight to a batch, and writes each of
-// them twice into its group's 8 positions.  The two halves of the group then
-// work on the same nonzeros, each lane on its own slice, and after 4 of the 8
-// steps one more exchange between the halves completes the dot products.
-#include <hip/hip_runtime.h>
-#include <utility>
+// Tile kernel variants: which (lanes per nonzero, float4 per lane) pair serves a rank, and
+// the table of instantiations (compiled in kernels_tile_p*.hip from kernels_tile_impl.hpp).
 #include "kernels.hpp"
-
-using namespace sddmm;
-
-namespace {
-
-typedef float vec4f __attribute__((ext_vector_type(4)));  // a plain vector: loadable through an LDS-qualified pointer
-
-__device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float acc)
-{
-    acc = fmaf(a.x, b.x, acc);
-    acc = fmaf(a.y, b.y, acc);
-    acc = fmaf(a.z, b.z, acc);
-    acc = fmaf(a.w, b.w, acc);
-    return acc;
-}
-
-// Two ways to walk a group's G nonzeros.
-// XORDER (H tile in LDS, rows a multiple of 256 bytes): lane l works, in its step
-// I, on the group's nonzero I ^ l, so acc[I] of lane l holds lane l's share of
-// nonzero I ^ l.  Every halving step adds to acc[j] the acc[j + S] of the lane S
-// away, which belongs to the same nonzero; after the last step acc[0] of lane l is
-// the whole dot product of nonzero l.  No lane ever has to choose which of two
-// registers to keep and which to send.  (The lanes of a group then read G
-// different H rows in one instruction: free in LDS, where only banks count.)
-// Otherwise all lanes of a group work on nonzero I in step I and read one
-// contiguous piece of its H row (what global memory wants), and each halving
-// step selects per lane what to keep and what to send.
-// v of lane (lane ^ X).  Distances below 8 are built from DPP lane selects (VALU,
-// and the compiler folds them into the add that uses the value): the LDS pipe, which
-// a ds_swizzle would occupy, is what the H-tile reads need.
-template <int X>
-__device__ __forceinline__ int from_lane_xor(int v)
-{
-    constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kQuadXor3 = 0x1B, kHalfMirror = 0x141;  // dpp_ctrl
-    if constexpr (X == 0) return v;
-    else if constexpr (X == 1) return __builtin_amdgcn_mov_dpp(v, kQuadXor1, 0xf, 0xf, true);
-    else if constexpr (X == 2) return __builtin_amdgcn_mov_dpp(v, kQuadXor2, 0xf, 0xf, true);
-    else if constexpr (X == 3) return __builtin_amdgcn_mov_dpp(v, kQuadXor3, 0xf, 0xf, true);
-    else if constexpr (X == 7) return __builtin_amdgcn_mov_dpp(v, kHalfMirror, 0xf, 0xf, true);  // lane ^ 7 inside 8 lanes
-    else if constexpr (X < 8)  // lane ^ X = (lane ^ 7) ^ (X ^ 7)
-        return __builtin_amdgcn_mov_dpp(__builtin_amdgcn_mov_dpp(v, kHalfMirror, 0xf, 0xf, true),
-                                        X == 4 ? kQuadXor3 : X == 5 ? kQuadXor2 : kQuadXor1, 0xf, 0xf, true);
-    else return __builtin_amdgcn_ds_swizzle(v, (X << 10) | 0x1f);
-}
-
-template <int G, int I, bool XORDER>
-__device__ __forceinline__ int column_of_step(int v)
-{
-    if constexpr (XORDER) return from_lane_xor<I>(v);
-    else return __builtin_amdgcn_ds_swizzle(v, (I << 5) | (0x1f & ~(G - 1)));  // from lane (lane & ~(G-1)) | I
-}
-
-// out[I] = (col of the lane this lane serves in step I) + base, for all G steps.
-// With the lane-permuted order and G = 8 or 4 each is ONE v_add_u32 with a DPP lane
-// select on its first operand (plus one v_mov for the half-mirrored copy that steps
-// 4-6 start from).  Written out because the compiler, left alone, keeps the select
-// and the add apart.  Plain VALU instructions only; the leading s_nop covers the two
-// wait states a DPP read needs after a VALU write of the same register.
-template <int G, bool XORDER>
-__device__ __forceinline__ void columns_of_steps(int col, int base, int (&out)[G])
-{
-    if constexpr (XORDER && G == 8) {
-        int hm;
-        out[0] = col + base;
-        asm("s_nop 1\n\t"
-            "v_mov_b32_dpp %[hm], %[c] row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r1], %[c], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r2], %[c], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r3], %[c], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r7], %[c], %[b] row_half_mirror row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r4], %[hm], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r5], %[hm], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r6], %[hm], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1"
-            : [hm] "=&v"(hm), [r1] "=&v"(out[1]), [r2] "=&v"(out[2]), [r3] "=&v"(out[3]), [r4] "=&v"(out[4]),
-              [r5] "=&v"(out[5]), [r6] "=&v"(out[6]), [r7] "=&v"(out[7])
-            : [c] "v"(col), [b] "v"(base));
-    } else if constexpr (XORDER && G == 4) {
-        out[0] = col + base;
-        asm("s_nop 1\n\t"
-            "v_add_u32_dpp %[r1], %[c], %[b] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r2], %[c], %[b] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
-            "v_add_u32_dpp %[r3], %[c], %[b] quad_perm:[3,2,1,0] row_mask:0xf bank_mask:0xf bound_ctrl:1"
-            : [r1] "=&v"(out[1]), [r2] "=&v"(out[2]), [r3] "=&v"(out[3])
-            : [c] "v"(col), [b] "v"(base));
-    } else {
-        [&]<int... I>(std::integer_sequence<int, I...>) {
-            ((void)(out[I] = column_of_step<G, I, XORDER>(col) + base), ...);
-        }(std::make_integer_sequence<int, G>{});
-    }
-}
-
-template <int S>
-__device__ __forceinline__ float xor_lane(float v)
-{
-    return __int_as_float(from_lane_xor<S>(__float_as_int(v)));
-}
-
-// XORDER: lane distance 1 first and the largest last, when one register is left:
-// distances 1 and 2 are one v_add with a DPP operand, larger ones cost more.
-template <int G, bool XORDER, int S = XORDER ? 1 : G / 2>
-__device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
-{
-    if constexpr (XORDER) {
-        if constexpr (S < G) {
-#pragma unroll
-            for (int j = 0; j < G; j += 2 * S) acc[j] += xor_lane<S>(acc[j + S]);
-            transpose_reduce_step<G, XORDER, S * 2>(acc, l);
-        }
-    } else if constexpr (S >= 1) {
-        const bool upper = (l & S) != 0;
-#pragma unroll
-        for (int j = 0; j < S; ++j) {
-            float keep = upper ? acc[j + S] : acc[j];
-            float send = upper ? acc[j] : acc[j + S];
-            acc[j] = keep + xor_lane<S>(send);
-        }
-        transpose_reduce_step<G, XORDER, S / 2>(acc, l);
-    }
-}
-
-// VMODE: where S.val comes from -- 0: a.sval (stream order), 1: a.val (sorted
-// order, read through the position), 2: nowhere (no scaling); 3 and 4: as 0 and 1
-// with the residual epilogue, out = val - dot (K slices after the first: out -= dot,
-// no value needed).
-//
-// The loop is software-pipelined by hand and free of branches around loads, so
-// that every wait is for exactly the data needed: while batch b is computed,
-// the index data of batch b+2 and the W row slice of batch b+1 are in flight.
-// GATHER: no LDS tile; scol holds the column and H rows are read from global
-// memory (the stream is then one unit in row order, for rows too short to tile).
-template <int G, int KPL, int VMODE, int NW, bool GATHER, bool ACC>
-__global__ __launch_bounds__(NW * 64)
-void sddmm_tile_kernel(const TileArgs a)
-{
-    extern __shared__ float4 lds_tile[];
-    constexpr int K4 = G * KPL;
-    constexpr bool RESIDUAL = VMODE >= 3;
-    constexpr bool STREAM_VAL = VMODE == 0 || (VMODE == 3 && !ACC);  // values read in stream order
-    constexpr bool SORTED_VAL = VMODE == 1 || (VMODE == 4 && !ACC);  // values read through the position
-    constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
-    constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
-    constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
-    // SHORTS: a batch may be marked "short" in a.btype: each of its groups then holds at most G/2
-    // nonzeros in its first G/2 positions and the same ones again in the other G/2.  With the
-    // lane-permuted order the upper half of the lanes then works on the same nonzeros as the lower
-    // half, each lane on its own slice, and steps G/2 .. G-1 can be left out: after G/2 steps every
-    // half group holds half of each dot product, and one more exchange adds the two.
-    constexpr bool SHORTS = tile_variant_shorts(G, KPL, GATHER);
-    // Groups that share one 16-lane LDS access phase read the 16-byte pieces of
-    // their rows in different orders (piece j ^ rot instead of j), so that their
-    // reads fall into different banks whenever rows are a multiple of 256 bytes
-    // apart.  NB distinct orders need NB base addresses per row; piece j is then
-    // at base[j % NB] + j*G*16, a compile-time offset.
-    constexpr int PHASE_GROUPS = (16 / G) >= 1 ? (16 / G) : 1;
-    constexpr int NB = GATHER ? 1 : (PHASE_GROUPS < KPL ? PHASE_GROUPS : KPL);
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: loop bounds stay in SGPRs
-    const int l = lane & (G - 1);
-    const int rot = (lane / G) & (NB - 1);
-
-    int slot[KPL];      // float4 index inside a row of lane's piece j
-    int lane_off[NB];   // byte offset of base t relative to the row start
-#pragma unroll
-    for (int j = 0; j < KPL; ++j) slot[j] = (j ^ rot) * G + l;
-#pragma unroll
-    for (int t = 0; t < NB; ++t) lane_off[t] = (l + ((t ^ rot) - t) * G) * 16;
-    // LDS addresses are kept as 32-bit integers: the address of this lane's first piece of
-    // an H row is (the row's offset in the tile) + lane_base0, added as soon as the offset arrives
-    using lds_f4_ptr = const __attribute__((address_space(3))) vec4f *;
-    const int lds_base = (int)(uint32_t)(uintptr_t)(lds_f4_ptr)reinterpret_cast<const vec4f *>(lds_tile);
-    const int lane_base0 = GATHER ? 0 : lds_base + lane_off[0];
-    int base_step[NB];  // base t of a row = base 0 + base_step[t]
-#pragma unroll
-    for (int t = 0; t < NB; ++t) {
-        base_step[t] = lane_off[t] - lane_off[0];
-        asm("" : "+v"(base_step[t]));  // one register, not an expression to be re-associated with each use
-    }
-
-    // this launch covers K elements [k_off, k_off + 4*K4) of rows that are row_k4 float4 long
-    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
-    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
-    const int row_k4 = a.K >> 2;
-
-    // This workgroup's share of the stream: either the items b, b + grid, ... of an item
-    // list (each inside one tile), or an equal, 64-aligned range of positions walked unit by unit.
-    int lo = 0, hi = 0, unit = 0, n_steps;
-    if (a.items) {
-        n_steps = (a.n_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    } else {
-        const int64_t total = a.unit_ptr[a.n_units];
-        lo = (int)(((total * blockIdx.x / gridDim.x) + 63) & ~(int64_t)63);
-        hi = (blockIdx.x + 1 == gridDim.x) ? (int)total
-                                           : (int)(((total * (blockIdx.x + 1) / gridDim.x) + 63) & ~(int64_t)63);
-        int a0 = 0, a1 = a.n_units;  // first unit whose end lies beyond lo
-        while (a0 < a1) {
-            const int mid = (a0 + a1) >> 1;
-            if (a.unit_ptr[mid + 1] <= lo) a0 = mid + 1; else a1 = mid;
-        }
-        unit = a0;
-        n_steps = 0;
-        for (int u = unit; u < a.n_units && a.unit_ptr[u] < hi; ++u) ++n_steps;
-    }
-    int cur_tile = -1;
-    for (int step = 0; step < n_steps; ++step) {
-        int begin, end, tile;
-        int type_base = 0;                     // index of the item's first batch in a.btype
-        // (constant address space: nothing writes the bits while the kernel runs, and only for such
-        // memory does the compiler use scalar loads next to the kernel's own stores)
-        using const_u32_ptr = const __attribute__((address_space(4))) uint32_t *;
-        const_u32_ptr types = nullptr;         // null: no short batches
-        if (a.items) {
-            const WorkItem wi = a.items[blockIdx.x + step * gridDim.x];
-            begin = wi.begin; end = wi.end; tile = wi.tile;
-            if (SHORTS) { type_base = wi.batch_base; types = (const_u32_ptr)(uintptr_t)a.btype; }
-        } else {
-            begin = max(lo, a.unit_ptr[unit + step]); end = min(hi, a.unit_ptr[unit + step + 1]);
-            tile = GATHER ? 0 : a.unit_tile[unit + step];
-        }
-        if (end <= begin) continue;
-        if (!GATHER && tile != cur_tile) {
-            if (cur_tile >= 0) __syncthreads();  // everyone is done with the previous tile
-            cur_tile = tile;
-            const int tile_base = tile * a.tile_x;
-            const int rows = min(a.tile_x, a.n_cols - tile_base);
-            const float4 *src = H4 + (size_t)tile_base * row_k4;
-            const int n4 = rows * K4;
-            for (int i = threadIdx.x; i < n4; i += NW * 64) {
-                const int r = i / K4, q = i - r * K4;
-                lds_tile[i] = src[(size_t)r * row_k4 + q];
-            }
-            __syncthreads();
-        }
-        const int nb = (end - begin + 63) >> 6;
-        // (the division runs on the vector unit; the results are uniform and go back to scalar
-        // registers, so that the batch counter and the batch type bits are scalar work)
-        const int b0 = __builtin_amdgcn_readfirstlane((int)((int64_t)nb * wave / NW));
-        const int b1 = __builtin_amdgcn_readfirstlane((int)((int64_t)nb * (wave + 1) / NW));
-        if (b0 >= b1) continue;  // (no barrier below this point inside the tile)
-        const int bf = min(b1, (end - begin) >> 6);  // [b0, bf): this wave's batches of 64 whole positions
-
-        // index data of one batch; positions past the item are clamped to its last
-        // one (and repeat its work), so no load sits behind a branch
-        // Index data of one batch.  The arrays are addressed as (uniform base of the
-        // item) + (32-bit byte offset of the lane), the form that needs no per-lane
-        // 64-bit arithmetic, and no load sits behind a branch.
-        struct Meta { uint32_t wrow, p; int col; float sv, old; };
-        const uint32_t last = (uint32_t)(end - begin - 1);
-        const char *perm_b = reinterpret_cast<const char *>(COMPACT ? a.pbase + begin / G : a.perm + begin);
-        const char *scol_b = COMPACT ? reinterpret_cast<const char *>(a.scol16 + begin)
-                                     : reinterpret_cast<const char *>(a.scol + begin);
-        const char *sval_b = reinterpret_cast<const char *>(a.sval + begin);
-        const char *grow_b = reinterpret_cast<const char *>(a.grow + begin / G);
-        // Steady state: batches are requested in order, two ahead of the one computed,
-        // with running offsets and no clamp (the batch after a wave's last one is
-        // requested and dropped; the arrays have readable slack behind the last position).
-        uint32_t o4 = ((uint32_t)(b0 << 6) + (uint32_t)lane) << 2;         // perm, scol, sval
-        uint32_t og = (((uint32_t)(b0 << 6) + (uint32_t)lane) / G) << 2;   // grow
-        auto issue_meta = [&]() -> Meta {
-            Meta m;
-            if constexpr (COMPACT) {
-                const uint32_t g = *reinterpret_cast<const uint32_t *>(grow_b + og);
-                m.wrow = g & ~(uint32_t)(G - 1);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + og) + min((uint32_t)l, g & (uint32_t)(G - 1));
-                m.col = (int)*reinterpret_cast<const uint16_t *>(scol_b + (o4 >> 1)) << ROW_SHIFT;
-            } else {
-                m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + og);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
-                m.col = *reinterpret_cast<const int *>(scol_b + o4);
-            }
-            m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
-            o4 += 256;
-            og += 256 / G;
-            return m;
-        };
-        // an item's last, partial batch: positions past the end are clamped to the last one
-        auto issue_meta_tail = [&](int bi) -> Meta {
-            const uint32_t t4 = min((uint32_t)(bi << 6) + (uint32_t)lane, last) << 2;
-            Meta m;
-            const uint32_t tg = (t4 / (4 * G)) << 2;
-            if constexpr (COMPACT) {
-                const uint32_t g = *reinterpret_cast<const uint32_t *>(grow_b + tg);
-                m.wrow = g & ~(uint32_t)(G - 1);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + tg) + min((t4 >> 2) & (uint32_t)(G - 1), g & (uint32_t)(G - 1));
-                m.col = (int)*reinterpret_cast<const uint16_t *>(scol_b + (t4 >> 1)) << ROW_SHIFT;
-            } else {
-                m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + tg);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + t4);
-                m.col = *reinterpret_cast<const int *>(scol_b + t4);
-            }
-            m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
-            return m;
-        };
-        // ACC (K slices after the first): the previous slices' partial result, requested
-        // one batch ahead of its use
-        auto issue_old = [&](Meta &m) { m.old = ACC ? a.out[GATHER ? (m.p & 0x7fffffffu) : m.p] : 0.f; };
-        // wrow: float4 index of the row's first element in W
-        auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
-            const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
-            wbase[0] = W4 + (wrow + (uint32_t)slot[0]);
-#pragma unroll
-            for (int t = 1; t < NB; ++t) wbase[t] = wbase[0] + (slot[t] - slot[0]);
-#pragma unroll
-            for (int j = 0; j < KPL; ++j) w[j] = wbase[j % NB][(j - j % NB) * G];
-        };
-        float pend_v;  // result of the batch before, not yet stored
-        uint32_t pend_p;
-        // (gather form: a position whose index carries bit 31 is padding that worked on
-        // another row's column; its result goes to a scratch line instead of the output)
-        auto flush = [&]() {
-            if constexpr (GATHER) {
-                float *dst = (int32_t)pend_p < 0 ? a.sink + (((blockIdx.x & 255) << 6) + lane) : a.out + pend_p;
-                *dst = pend_v;
-            } else {
-                a.out[pend_p] = pend_v;
-            }
-        };
-        // c[I]: where the H row this lane works on in step I starts (LDS: byte address of
-        // this lane's first piece; gather form: float4 index of the row); cn: the same for the next batch, requested here after the last LDS
-        // read so that the latency hides behind the reduction
-        auto compute = [&]<bool SHORT>(std::bool_constant<SHORT>, const float4 (&w)[KPL], const Meta &m, const int (&c)[G],
-                                       int (&cn)[G], int next_col) {
-            constexpr int STEPS = SHORT ? G / 2 : G;
-            float v = m.sv;
-            if (SORTED_VAL) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
-            float acc[STEPS];
-            [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)[&] {
-                    float s = 0.f;
-                    if constexpr (GATHER) {
-                        const float4 *hr = H4 + (uint32_t)c[I];  // scol: float4 index of the H row
-                        float4 h[KPL];
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) h[j] = hr[slot[j]];
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) s = dot4(w[j], h[j], s);
-                    } else {
-                        int base[NB];  // c[I] is base 0 already
-                        base[0] = c[I];
-#pragma unroll
-                        for (int t = 1; t < NB; ++t) base[t] = c[I] + base_step[t];
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) {
-                            const vec4f h = *(lds_f4_ptr)(uintptr_t)(uint32_t)(base[j % NB] + j * G * 16);
-                            s = dot4(w[j], make_float4(h.x, h.y, h.z, h.w), s);
-                        }
-                    }
-                    acc[I] = s;
-                }(), ...);
-            }(std::make_integer_sequence<int, STEPS>{});
-            columns_of_steps<G, XORDER>(next_col, lane_base0, cn);
-            if constexpr (SHORT) {
-                transpose_reduce_step<G / 2, XORDER>(acc, l);  // inside each half group
-                acc[0] += xor_lane<G / 2>(acc[0]);             // the other half's slices of the same nonzero
-            } else {
-                transpose_reduce_step<G, XORDER>(acc, l);
-            }
-            // The store is left to the start of the next batch (flush): issued here it
-            // would sit, unfinished, in front of the loads that batch waits for.  In a
-            // whole batch it needs no predicate: a padding position repeats a nonzero of
-            // its own group and so writes that nonzero's own result a second time.
-            if constexpr (RESIDUAL) pend_v = ACC ? m.old - acc[0] : v - acc[0];
-            else pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
-            pend_p = m.p;
-        };
-
-        // the type bits of 32 consecutive batches, held in scalar registers
-        uint32_t type_word = 0;
-        int type_at = -1;
-        auto short_batch = [&](int b) -> bool {
-            if constexpr (!SHORTS) return false;
-            if (!types) return false;
-            const int g = type_base + b;
-            if ((g >> 5) != type_at) { type_at = g >> 5; type_word = types[type_at]; }
-            return (type_word >> (g & 31)) & 1u;
-        };
-        auto run = [&](int b, const float4 (&w)[KPL], const Meta &m, const int (&c)[G], int (&cn)[G], int next_col) {
-            if (short_batch(b)) compute(std::true_type{}, w, m, c, cn, next_col);
-            else compute(std::false_type{}, w, m, c, cn, next_col);
-        };
-
-        float4 wa[KPL], wb[KPL];
-        int ca[G], cb[G];
-        if (b0 < bf) {
-            Meta m0 = issue_meta();
-            Meta m1 = issue_meta();
-            issue_old(m0);
-            issue_w(wa, m0.wrow);
-            columns_of_steps<G, XORDER>(m0.col, lane_base0, ca);
-            Meta m2 = issue_meta();
-            issue_old(m1);
-            issue_w(wb, m1.wrow);
-            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
-            run(b0, wa, m0, ca, cb, m1.col);
-            for (int bi = b0 + 1; bi < bf; bi += 2) {
-                flush();
-                Meta m3 = issue_meta();
-                issue_old(m2);
-                issue_w(wa, m2.wrow);
-                __builtin_amdgcn_sched_barrier(0);
-                run(bi, wb, m1, cb, ca, m2.col);
-                if (bi + 1 >= bf) break;
-                flush();
-                Meta m4 = issue_meta();
-                issue_old(m3);
-                issue_w(wb, m3.wrow);
-                __builtin_amdgcn_sched_barrier(0);
-                run(bi + 1, wa, m2, ca, cb, m3.col);
-                m1 = m3;
-                m2 = m4;
-            }
-            flush();
-        }
-        if (bf < b1) {
-            // the item's last, partial batch: lanes past its end work on the last
-            // position once more and store nothing
-            Meta mt = issue_meta_tail(bf);
-            issue_old(mt);
-            issue_w(wa, mt.wrow);
-            columns_of_steps<G, XORDER>(mt.col, lane_base0, ca);
-            compute(std::false_type{}, wa, mt, ca, cb, mt.col);
-            if (begin + (bf << 6) + lane < end) flush();
-        }
-    }
-}
-
-}  // namespace
 
 namespace sddmm {
 
@@ -470,24 +17,22 @@ TileVariant pick_tile_variant(int K, int want_g)
     return best;
 }
 
+TileFn tile_kernel_part0(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+TileFn tile_kernel_part1(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+TileFn tile_kernel_part2(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+TileFn tile_kernel_part3(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+
+// vmode: see the kernel template (where S.val comes from, which epilogue)
 TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
 {
-#define SDDMM_PICK_NW(g, kpl, vm, nw)                                                                       \
-    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, false, true>                    \
-                : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
-#define SDDMM_PICK(g, kpl, vm)                                                                              \
-    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), 4, true, true>            \
-                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
-            : (nwaves == 12 ? SDDMM_PICK_NW(g, kpl, vm, 12) : SDDMM_PICK_NW(g, kpl, vm, 16)))
-#define SDDMM_CASE(g, kpl)                                                                                  \
-    if (v.G == g && v.KPL == kpl)                                                                           \
-        return vmode == 0 ? SDDMM_PICK(g, kpl, 0) : vmode == 1 ? SDDMM_PICK(g, kpl, 1) : vmode == 2 ? SDDMM_PICK(g, kpl, 2)      \
-             : vmode == 3 ? SDDMM_PICK(g, kpl, 3) : SDDMM_PICK(g, kpl, 4);
-    SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
-    SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
-#undef SDDMM_CASE
-#undef SDDMM_PICK
-#undef SDDMM_PICK_NW
+    switch (vmode) {
+    case 0: return tile_kernel_part0(v, vmode, gather, accumulate, nwaves);
+    case 1: return tile_kernel_part1(v, vmode, gather, accumulate, nwaves);
+    case 2: return tile_kernel_part2(v, vmode, gather, accumulate, nwaves);
+    case 3: return tile_kernel_part3(v, vmode, gather, accumulate, nwaves);
+    case 4: return tile_kernel_part4(v, vmode, gather, accumulate, nwaves);
+    }
     return nullptr;
 }
 

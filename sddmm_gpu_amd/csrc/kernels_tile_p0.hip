@@ -1,0 +1,28 @@
+// Tile kernels, part 0: the instantiations for value mode 0 (out = val * dot, values in stream order).
+// The kernel template is compiled in several translation units side by side, which
+// divides the build time of the slowest file.
+#include "kernels_tile_impl.hpp"
+
+namespace sddmm {
+
+TileFn tile_kernel_part0(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
+{
+#define SDDMM_PICK_NW(g, kpl, vm, nw)                                                                       \
+    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, false, true>                    \
+                : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
+#define SDDMM_PICK(g, kpl, vm)                                                                              \
+    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), 4, true, true>            \
+                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
+            : (nwaves == 12 ? SDDMM_PICK_NW(g, kpl, vm, 12) : SDDMM_PICK_NW(g, kpl, vm, 16)))
+#define SDDMM_CASE(g, kpl)                                                                                  \
+    if (v.G == g && v.KPL == kpl)                                                                           \
+        return SDDMM_PICK(g, kpl, 0);
+    SDDMM_CASE(4, 2) SDDMM_CASE(4, 4) SDDMM_CASE(4, 8) SDDMM_CASE(8, 1) SDDMM_CASE(8, 2) SDDMM_CASE(8, 4) SDDMM_CASE(8, 8)
+    SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
+#undef SDDMM_CASE
+#undef SDDMM_PICK
+#undef SDDMM_PICK_NW
+    return nullptr;
+}
+
+}  // namespace sddmm
