@@ -61,6 +61,32 @@ def test_full_size(oracle, cfg, K):
     assert torch.equal(outp, out)
     del outp
 
+    # (1c) the fused residual epilogue val - dot: the sample against the oracle (whose residual
+    # form is val minus its scaled form with val = 1, bit for bit), and every nonzero against
+    # val minus the GPU's own unscaled dot product (the same sums; only the last rounding and,
+    # with K slices, the order of the subtractions differ)
+    plan = capi.Plan.from_device_csr(n_rows, n_cols, nnz, d["row_ptr"].data_ptr(), d["col_ind"].data_ptr(), K, 0, 0,
+                                     capi.KERNEL_AUTO)
+    stream = torch.cuda.current_stream().cuda_stream
+    dot = torch.empty(nnz, device=dev); res = torch.empty(nnz, device=dev)
+    plan.execute(0, d["W"].data_ptr(), d["H"].data_ptr(), dot.data_ptr(), stream)            # no values: out = dot
+    plan.execute_epilogue(d["val"].data_ptr(), d["W"].data_ptr(), d["H"].data_ptr(), res.data_ptr(),
+                          capi.EPILOGUE_RESIDUAL, stream)
+    torch.cuda.synchronize()
+    plan.close()
+    # (the partial dot products of the K slices can be larger than their sum: Cauchy-Schwarz bounds them)
+    wn = torch.linalg.vector_norm(d["W"], dim=1); hn = torch.linalg.vector_norm(d["H"], dim=1)
+    slack = 2.0 ** -22 * (d["val"].abs() + wn[d["row_ind"].long()] * hn[d["col_ind"].long()]) * max(1, K // 128)
+    del wn, hn
+    assert bool(((res - (d["val"] - dot)).abs() <= slack).all())
+    W = d["W"].cpu().numpy(); H = d["H"].cpu().numpy()
+    cpu_dot = oracle.sddmm_coo(rows, cols, np.ones_like(vals), W, H)
+    _, absp1 = oracle.sddmm_f64(rows, cols, np.ones_like(vals), W, H)
+    cpu_res = vals - cpu_dot
+    lim = 1e-5 * np.sqrt(K) * np.maximum(np.abs(cpu_dot), absp1 / 100.0) + 2.0 ** -23 * np.abs(cpu_res)
+    assert not (np.abs(res[idx].cpu().numpy().astype(np.float64) - cpu_res) > lim).any()
+    del W, H, dot, res
+
     # (2) scaling W by a power of two scales every output exactly
     out4, _ = run(d, capi.KERNEL_AUTO, W=d["W"] * 4.0)
     assert torch.equal(out4, out * 4.0)
