@@ -630,6 +630,23 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                         const int32_t j = nt >= per_die ? deal[(size_t)die * nt + (size_t)step * per_die + slot] : slot % nt;
                         items.push_back(item_of(sh, j));
                     }
+            } else if (shares == 1 && c.cus % 8 == 0 && (int64_t)tiles_ne.size() > c.cus &&
+                       env_i64("SDDMM_TILE_RUNS", 1) != 0) {
+                // More tiles than workgroups (a wide matrix; one item per tile, all rows).  Neighbouring
+                // tiles of a banded matrix share most of their rows: each turn gives a run of
+                // consecutive tiles to the workgroups of one die (workgroup b runs on die b % 8), so
+                // that a W row is fetched into one L2 for all the tiles that need it in that turn,
+                // instead of into every die's.  Banded 2^20, K=512: 6.63 -> 5.29 ms, reads across
+                // the L2 boundary 44 -> 29.5 GB per step.  (Cutting the rows into blocks that fit L2
+                // as well, all workgroups of a die on the same block, was slower, 7.7-10.7 ms: the
+                // items get small and every one stages its H tile again.)
+                const int per_die = c.cus / 8;
+                const int64_t n = (int64_t)tiles_ne.size(), turns = (n + c.cus - 1) / c.cus;
+                for (int64_t step = 0; step < turns; ++step)
+                    for (int b = 0; b < c.cus; ++b) {
+                        const int64_t idx = step * c.cus + (int64_t)(b % 8) * per_die + b / 8;
+                        items.push_back(idx < n ? item_of(0, tiles_ne[(size_t)idx]) : WorkItem{0, 0, 0, 0});
+                    }
             } else {
                 for (int sh = 0; sh < shares; ++sh)
                     for (int32_t j : tiles_ne) items.push_back(item_of(sh, j));
