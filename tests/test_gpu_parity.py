@@ -297,6 +297,40 @@ def test_residual_epilogue_needs_values():
     assert e.value.code == capi.ERR_ARG
 
 
+@pytest.mark.parametrize("K", [64, 256])
+def test_execute_can_be_captured_in_a_graph(oracle, monkeypatch, K):
+    """sddmm_execute only launches kernels on the caller's stream (no allocation, no
+    memset, no synchronisation), so a caller may record it into a HIP graph.  The graph
+    is replayed several times with eager work and synchronisations in between and with
+    W changed in place; every replay must give the eager result's bits."""
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # the split plan: two launches per K slice
+    d = synth.make(3, 0.05, K=K, seed=31)
+    dev = torch.device("cuda:0")
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    plan = S.plan(K, 0, 0, capi.KERNEL_AUTO)
+    W = d["W"].to(dev).contiguous(); H = d["H"].to(dev).contiguous()
+    out = torch.zeros(d["nnz"], device=dev); eager = torch.zeros(d["nnz"], device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), side.cuda_stream)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        W.mul_(2.0 if rep else 1.0)          # eager work between the replays
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        plan.execute(0, W.data_ptr(), H.data_ptr(), eager.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+    d2 = dict(d); d2["W"] = d["W"] * 4.0
+    check(d2, out.cpu().numpy(), oracle, K=K)
+
+
 def test_device_plan_rejects_bad_csr():
     dev = torch.device("cuda:0")
     rp = torch.tensor([0, 2, 3], dtype=torch.int32, device=dev)
