@@ -222,7 +222,10 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
     a.seg_row = d_seg_row; a.perm = d_perm; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
     L.perm = d_perm;
     a.nnz = (int32_t)n;
-    a.chunk = 64 * kRowGatherBatchesPerWave * (kRowGatherBlock / 64);
+    // nonzeros per workgroup: up to 8 batches of 64 per wave, fewer when that would leave compute units idle
+    const int64_t waves_wanted = 2 * (int64_t)c.cus * (kRowGatherBlock / 64);
+    const int per_wave = (int)std::clamp<int64_t>(n / (64 * waves_wanted), 1, kRowGatherBatchesPerWave);
+    a.chunk = 64 * per_wave * (kRowGatherBlock / 64);
     a.K = c.K; a.n_cols = (int32_t)c.n_cols; a.tile_x = (int32_t)c.n_cols;
     a.generic_perm = var.G == 0;
     L.grid = (int32_t)((n + a.chunk - 1) / a.chunk);
@@ -365,7 +368,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 const int64_t nt = (c.n_cols + x - 1) / x;
                 shares = (int)(c.cus / nt);
                 const int64_t per_die = c.cus / 8;
-                if (assign == 2 && c.cus % 8 == 0 && nt == n2 && (n2 % per_die == 0 || per_die % n2 == 0)) {
+                // (every row block stages every H tile again: with few nonzeros per tile -- less than
+                // twice a tile's bytes in index data -- the assignment with the fewest row blocks wins)
+                const bool staging_dominates = 8.0 * (double)nt * x * ks * 4 > 2.0 * 12.5 * (double)L.nnz;
+                if (assign == 2 && c.cus % 8 == 0 && nt == n2 && (n2 % per_die == 0 || per_die % n2 == 0) &&
+                    !(staging_dominates && env_i64("SDDMM_TILE_FEW_BLOCKS", 1) != 0)) {
                     xcd_local = true;
                     xcd_steps = (int)std::max<int64_t>(1, n2 / per_die);
                     shares = 8 * (int)std::max<int64_t>(1, per_die / n2);
