@@ -241,6 +241,26 @@ int sddmm_execute_profiled(const sddmm_plan *plan, const float *d_val, const flo
 int sddmm_gpu(const sddmm_plan *plan, const float *h_W, const float *h_H, float *h_out,
               float *kernel_ms);
 
+/* Plan-free SDDMM over a CSR pattern in device memory that allocates nothing:
+ * no hipMalloc / hipFree and no allocating library routine on any call.  It has
+ * no counterpart in the reference (whose sddmm_GPU allocates and frees on every
+ * call, sddmm.cu:38-73, 147-150); it is for callers that cannot allocate --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc -- and therefore cannot create a plan.  Same result as
+ * sddmm_plan_create_device(..., SDDMM_KERNEL_ROW_GATHER) + sddmm_execute, bit
+ * for bit: the row-gather kernel, whose per-batch side array (the row of every
+ * 64th nonzero) is built on the device, on `stream`, into a fixed 16 MiB
+ * device array of the library.  All pointers are device pointers; d_val may be
+ * NULL (out[p] = dot).  The pattern is not validated (that would need a copy
+ * to the host): d_row_ptr must be monotone with d_row_ptr[0] = 0 and
+ * d_row_ptr[n_rows] = nnz, columns inside [0, n_cols).  nnz above SDDMM_NOALLOC_MAX_NNZ is rejected with
+ * SDDMM_ERR_RANGE.  Every call on a GPU uses that GPU's one array: calls that
+ * overlap in time on the same GPU (different streams or threads) race.       */
+#define SDDMM_NOALLOC_MAX_NNZ (1 << 28)
+int sddmm_csr_noalloc(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                      const int32_t *d_col_ind, const float *d_val, int32_t K, const float *d_W,
+                      const float *d_H, float *d_out, void *stream);
+
 /* Number of visible devices and the gcnArchName of device 0 ("" if none). */
 int sddmm_device_info(int *n_devices, char *arch, int arch_len);
 

@@ -82,6 +82,8 @@ SIGNATURES = {
     "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
     "sddmm_execute_profiled": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(LaunchProfile), c_int32]),
     "sddmm_gpu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_float)]),
+    "sddmm_csr_noalloc": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p,
+                                  c_void_p, c_void_p]),
     "sddmm_device_info": (c_int, [POINTER(c_int), c_char_p, c_int]),
 }
 
@@ -293,6 +295,12 @@ def init_reference(n, k):
     X = np.empty((n, k), np.float32)
     check(lib().sddmm_init_reference(_np_ptr(X), n, k))
     return X
+
+
+def csr_noalloc(n_rows, n_cols, nnz, d_row_ptr, d_col_ind, d_val, K, d_W, d_H, d_out, stream=0):
+    """Plan-free SDDMM over a device CSR that allocates nothing (sddmm_csr_noalloc)."""
+    check(lib().sddmm_csr_noalloc(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), c_void_p(d_val or None), K,
+                                  c_void_p(d_W), c_void_p(d_H), c_void_p(d_out), c_void_p(stream or None)))
 
 
 def device_info():

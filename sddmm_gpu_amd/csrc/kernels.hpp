@@ -31,6 +31,12 @@ struct KArgs {
     int32_t n_cols;
     int32_t generic_perm;
     int32_t residual;          // 0: out = val * dot;  1: out = val - dot
+    // Plan-free form (batch_seg and batch_mask are null then): batch_row[b] is the row of stream
+    // position 64*b, and every lane finds its own row by a search of row_ptr between the
+    // rows of two consecutive batches.
+    const int32_t *row_ptr;    // [n_rows+1]
+    const int32_t *batch_row;  // [ceil(nnz/64)]
+    int32_t n_rows;
 };
 
 constexpr int kRowGatherBlock = 256;   // 4 waves

@@ -86,6 +86,25 @@ struct Batch {
     float v;
 };
 
+// Row (segment) of stream position pos, which lies in batch gb.  With the plan's side
+// arrays: the batch's first segment plus the number of segment starts up to this lane.
+// Plan-free form: the largest row r between the rows of this batch's and the next
+// batch's first positions with row_ptr[r] <= pos (empty rows in between never qualify
+// as the largest).
+__device__ __forceinline__ int segment_of(const KArgs &a, int gb, int pos, uint64_t le)
+{
+    if (a.batch_row) {
+        int lo = a.batch_row[gb];
+        int hi = (gb + 1 < ((a.nnz + 63) >> 6)) ? a.batch_row[gb + 1] : a.n_rows - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (a.row_ptr[mid] <= pos) lo = mid; else hi = mid - 1;
+        }
+        return lo;
+    }
+    return a.batch_seg[gb] + __popcll(a.batch_mask[gb] & le);
+}
+
 // K = 4 * (number of float4 per row); each lane of a group owns KPL float4
 // slots of a row: slot j sits at float4 index (((j + rot) % KPL) * G + l).  `rot`
 // differs between the groups that share one 16-lane LDS access phase, so that
@@ -154,7 +173,7 @@ void sddmm_stream_kernel(const KArgs a)
             const int pos = begin + (bi << 6) + lane;
             if (bi < b1 && pos < end) {
                 const int gb = batch_base + bi;
-                const int seg = a.batch_seg[gb] + __popcll(a.batch_mask[gb] & le);
+                const int seg = segment_of(a, gb, pos, le);
                 b.row = a.seg_row ? a.seg_row[seg] : seg;
                 b.p = a.perm ? a.perm[pos] : pos;
                 b.col = a.scol ? a.scol[pos] : a.col_ind[b.p];
@@ -244,12 +263,11 @@ void sddmm_generic_kernel(const KArgs a)
         const int pos = begin + (bi << 6) + lane;
         const bool valid = pos < end;
         const int gb = batch_base + bi;
-        const uint64_t mask = a.batch_mask[gb];
         const uint64_t le = (lane == 63) ? ~0ull : ((2ull << lane) - 1ull);
-        const int seg = a.batch_seg[gb] + __popcll(mask & le);
         int row = -1, col = 0, p = 0;
         float v = 0.f;
         if (valid) {
+            const int seg = segment_of(a, gb, pos, le);
             row = a.seg_row ? a.seg_row[seg] : seg;
             p = a.perm ? a.perm[pos] : pos;
             col = a.col_ind[p];
