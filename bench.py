@@ -86,7 +86,7 @@ def cpu_baseline(d, K, budget_s=12.0):
                 sample=f"first {n} of {nnz} nonzeros (rows in order), K={K}, best of 2 runs, {t * 1e3:.1f} ms")
 
 
-KERNEL_NAMES = {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid"}
+KERNEL_NAMES = {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid", 5: "dense_block"}
 
 
 def main():

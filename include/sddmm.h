@@ -44,7 +44,11 @@ enum {
     SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM */
     SDDMM_KERNEL_LDS_TILE = 2,   /* column tiles of H staged in LDS, W row (re)loaded per row run */
     SDDMM_KERNEL_PANEL = 3,      /* row panels of W resident in VGPRs, column tiles of H swept through LDS */
-    SDDMM_KERNEL_HYBRID = 4      /* rows split by length: long -> LDS_TILE, medium -> PANEL, short -> ROW_GATHER */
+    SDDMM_KERNEL_HYBRID = 4,     /* the dense core as DENSE_BLOCK launches, the rest split by row length: long rows ->
+                                    LDS_TILE, short rows -> ROW_GATHER (what AUTO builds) */
+    SDDMM_KERNEL_DENSE_BLOCK = 5 /* blocks of 128 heavy rows x 128 popular columns computed whole on the matrix cores,
+                                    their nonzeros picked from the result; never a plan of its own, only a launch of a
+                                    HYBRID plan (reported by sddmm_execute_profiled) */
 };
 
 typedef struct sddmm_coo sddmm_coo;   /* host-side sparse matrix (COO, int32/int32/fp32) */
@@ -70,6 +74,8 @@ typedef struct sddmm_plan_info {
     int64_t padded_positions; /* stream positions of the LDS_TILE launches, padding included */
     int64_t short_batches;    /* batches of 64 of those positions that run in half the steps */
     double plan_ms;       /* host time spent in the tiling pass + upload */
+    int64_t dense_nnz;    /* nonzeros handled by the DENSE_BLOCK launch */
+    int64_t dense_blocks; /* its 128 x 128 blocks */
 } sddmm_plan_info;
 
 const char *sddmm_last_error(void);
@@ -124,6 +130,17 @@ int sddmm_coo_compress_rows(const sddmm_coo *S, int32_t *row_ptr, int32_t *row_h
  * CLI runs with.  Replaces initial(), util.h:75-81.  X is a host pointer.   */
 int sddmm_init_reference(float *X, int64_t n, int32_t k);
 
+/* The SDDMM on the host cores: out[p] = S.val[p] * (sum over t ascending of
+ * W[row_p*K+t] * H[col_p*K+t]), every sum sequential in fp32 -- the arithmetic
+ * and the result, bit for bit, of sddmm_CPU_CSR / sddmm_CPU_COO
+ * (sddmm.cu:153-200); nonzeros are dealt to n_threads threads (<= 0: all
+ * cores), the counterpart of the reference's "#pragma omp parallel for" over
+ * rows.  S must be sorted; W, H, out are host pointers (out: nnz fp32).  Needs
+ * no GPU: this is what the command-line tool checks the device result
+ * against, as the reference does at sddmm.cu:126-145.                       */
+int sddmm_cpu(const sddmm_coo *S, int32_t K, const float *W, const float *H, float *out,
+              int32_t n_threads);
+
 /* --------------------------------------------------------------- tiling --- */
 
 /* Host-side result of the tiling pass, for inspection and tests.  S is cut
@@ -175,6 +192,60 @@ int sddmm_plan_create(const sddmm_coo *S, int32_t K, int32_t tile_size_x, int32_
 int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
                              const int32_t *d_col_ind, int32_t K, int32_t tile_size_x,
                              int32_t tile_size_y, uint32_t flags, sddmm_plan **out);
+
+/* Everything that shapes a plan, for callers that want more than the two tile
+ * sizes.  sddmm_plan_options_init() sets every field to "let the planner
+ * choose" (-1; kernel AUTO; tile sizes 0); a plan built from the same matrix, K
+ * and options is always the same plan.  Every field can also be overridden
+ * from the environment (variable named in brackets, read when a plan is
+ * created, unless ignore_env is set) -- a tuning aid for runs where the caller's
+ * code cannot be changed; sddmm_plan_get_options() reports the values a plan
+ * was actually built with, overrides included.
+ *
+ * tile_size_x is honoured by every LDS-tile launch (capped by what fits the
+ * 160 KB LDS).  tile_size_y is the row-panel height of the PANEL kernel and of
+ * an explicitly requested LDS_TILE plan; the plans AUTO/HYBRID build assign
+ * whole column tiles to workgroups and ignore it (plan_info.tile_size_y reports
+ * INT32_MAX there).                                                          */
+typedef struct sddmm_plan_options {
+    int32_t kernel;             /* SDDMM_KERNEL_*                                   [SDDMM_KERNEL]        */
+    int32_t tile_size_x;        /* columns of S per LDS tile, 0 = choose            [SDDMM_TILE_X]        */
+    int32_t tile_size_y;        /* row-panel height, 0 = choose                     [SDDMM_TILE_Y]        */
+    int32_t k_slice;            /* K elements per tile-kernel launch (32/64/128)    [SDDMM_TILE_KSLICE]   */
+    int32_t tile_lanes;         /* lanes per nonzero of the tile kernel (4/8/16)    [SDDMM_TILE_G]        */
+    int32_t tile_waves;         /* waves per workgroup of the tile kernel (12/16)   [SDDMM_TILE_WAVES]    */
+    int32_t tile_assign;        /* 0 equal position ranges, 1 tile x row block,
+                                   2 the same with a row block's tiles on one die   [SDDMM_TILE_ASSIGN]   */
+    int32_t tile_few_blocks;    /* 0/1 fewest row blocks when staging dominates     [SDDMM_TILE_FEW_BLOCKS] */
+    int32_t tile_short_batches; /* 0/1 run ends of <= lanes/2 nonzeros batched apart [SDDMM_TILE_SHORT]    */
+    int32_t tile_deal;          /* 0/1 heavy and light tiles dealt to one workgroup [SDDMM_TILE_DEAL]     */
+    int32_t tile_runs;          /* 0/1 runs of neighbouring tiles to one die        [SDDMM_TILE_RUNS]     */
+    int32_t gather_lanes;       /* lanes per nonzero of the short-row launch        [SDDMM_GATHER_G]      */
+    int32_t gather_padded;      /* 0/1 short rows through the padded gather kernel  [SDDMM_GATHER_PADDED] */
+    int32_t gather_sink;        /* 0/1 padding of that stream flagged and dropped   [SDDMM_GATHER_SINK]   */
+    int32_t row_padded;         /* 0/1 ROW_GATHER plans use the padded gather kernel [SDDMM_ROW_PADDED]    */
+    int32_t unpadded_tile;      /* 0/1 LDS_TILE plans use the unpadded stream kernel [SDDMM_UNPADDED_TILE] */
+    int32_t dense_blocks;       /* 0/1 dense core on the matrix cores (-1: by K)    [SDDMM_DENSE]         */
+    int32_t dense_permille;     /* least fill of a dense block, in 1/1000           [SDDMM_DENSE_PERMILLE] */
+    int32_t dense_rb_group;     /* row blocks swept together by one die             [SDDMM_DENSE_RB_GROUP] */
+    int32_t ignore_env;         /* 1: the environment is not consulted                                      */
+    int64_t dense_min_nnz;      /* fewer dense nonzeros than this: no dense launch  [SDDMM_DENSE_MIN_NNZ] */
+    int64_t panel_bytes;        /* W bytes per row panel of an LDS_TILE stream      [SDDMM_PANEL_BYTES]   */
+    int64_t short_row_max;      /* rows with fewer nonzeros go to the short class   [SDDMM_SHORT_ROW_MAX] */
+    int64_t stage_factor;       /* long class needs this many nonzeros per staged H row [SDDMM_STAGE_FACTOR] */
+    int64_t split_min_nnz;      /* smaller matrices are one launch                  [SDDMM_SPLIT_MIN_NNZ] */
+} sddmm_plan_options;
+void sddmm_plan_options_init(sddmm_plan_options *opt);
+
+/* sddmm_plan_create / sddmm_plan_create_device with the full option set
+ * (opt == NULL: defaults).  No counterpart in the reference, whose only knobs
+ * are the two tile sizes on the command line (sddmm.cu:253-254).             */
+int sddmm_plan_create_opt(const sddmm_coo *S, int32_t K, const sddmm_plan_options *opt,
+                          sddmm_plan **out);
+int sddmm_plan_create_device_opt(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                                 const int32_t *d_col_ind, int32_t K, const sddmm_plan_options *opt,
+                                 sddmm_plan **out);
+int sddmm_plan_get_options(const sddmm_plan *plan, sddmm_plan_options *opt);
 
 /* Gives the plan its own copy of S.val (nnz fp32 in sorted order, device
  * pointer), laid out the way each of its kernels streams the nonzeros, so
@@ -260,6 +331,13 @@ int sddmm_gpu(const sddmm_plan *plan, const float *h_W, const float *h_H, float 
 int sddmm_csr_noalloc(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
                       const int32_t *d_col_ind, const float *d_val, int32_t K, const float *d_W,
                       const float *d_H, float *d_out, void *stream);
+
+/* Measurement aid: copies n_bytes (a multiple of 16, both pointers 16-byte
+ * aligned device memory) with a plain streaming kernel, sddmm_copy_probe_kernel,
+ * on `stream`.  A profile of a run that also calls this holds a kernel of known
+ * size (n_bytes read, n_bytes written) to scale the HBM byte counters by.  No
+ * counterpart in the reference.                                              */
+int sddmm_copy_probe(const void *d_src, void *d_dst, int64_t n_bytes, void *stream);
 
 /* Number of visible devices and the gcnArchName of device 0 ("" if none). */
 int sddmm_device_info(int *n_devices, char *arch, int arch_len);

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsddmm_hip.so")
 
 OK, ERR_ARG, ERR_IO, ERR_FORMAT, ERR_RANGE, ERR_UNSORTED, ERR_HIP, ERR_NOMEM = range(8)
-KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL, KERNEL_HYBRID = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL, KERNEL_HYBRID, KERNEL_DENSE_BLOCK = 0, 1, 2, 3, 4, 5
 EPILOGUE_SCALE, EPILOGUE_RESIDUAL = 0, 1
 
 
@@ -33,10 +33,32 @@ class PlanInfo(C.Structure):
                 ("lanes_per_nnz", c_int32), ("lds_bytes", c_int32), ("grid", c_int32), ("block", c_int32),
                 ("n_blocks", c_int64), ("device_bytes", c_int64), ("class_nnz", c_int64 * 3), ("class_rows", c_int64 * 3), ("padded_positions", c_int64),
                 ("short_batches", c_int64),
-                ("plan_ms", c_double)]
+                ("plan_ms", c_double), ("dense_nnz", c_int64), ("dense_blocks", c_int64)]
 
     def as_dict(self):
         return {f: (list(getattr(self, f)) if f.startswith("class_") else getattr(self, f)) for f, _ in self._fields_}
+
+
+class PlanOptions(C.Structure):
+    """sddmm_plan_options; PlanOptions.defaults(**fields) starts from sddmm_plan_options_init."""
+    _fields_ = [(n, c_int32) for n in (
+        "kernel", "tile_size_x", "tile_size_y", "k_slice", "tile_lanes", "tile_waves", "tile_assign", "tile_few_blocks",
+        "tile_short_batches", "tile_deal", "tile_runs", "gather_lanes", "gather_padded", "gather_sink", "row_padded",
+        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "ignore_env")] + [(n, c_int64) for n in (
+        "dense_min_nnz", "panel_bytes", "short_row_max", "stage_factor", "split_min_nnz")]
+
+    @classmethod
+    def defaults(cls, **kw):
+        o = cls()
+        lib().sddmm_plan_options_init(byref(o))
+        for k, v in kw.items():
+            if k not in dict(cls._fields_):
+                raise KeyError(k)
+            setattr(o, k, v)
+        return o
+
+    def as_dict(self):
+        return {f: getattr(self, f) for f, _ in self._fields_}
 
 
 class LaunchProfile(C.Structure):
@@ -68,12 +90,18 @@ SIGNATURES = {
     "sddmm_coo_row_ptr": (c_int, [c_void_p, c_void_p]),
     "sddmm_coo_compress_rows": (c_int, [c_void_p, c_void_p, c_void_p, POINTER(c_int64)]),
     "sddmm_init_reference": (c_int, [c_void_p, c_int64, c_int32]),
+    "sddmm_cpu": (c_int, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32]),
     "sddmm_tiling_create": (c_int, [c_void_p, c_int32, c_int32, POINTER(c_void_p)]),
     "sddmm_tiling_get": (c_int, [c_void_p, POINTER(TilingView)]),
     "sddmm_tiling_destroy": (None, [c_void_p]),
     "sddmm_plan_create": (c_int, [c_void_p, c_int32, c_int32, c_int32, c_uint32, POINTER(c_void_p)]),
     "sddmm_plan_create_device": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                          c_uint32, POINTER(c_void_p)]),
+    "sddmm_plan_options_init": (None, [POINTER(PlanOptions)]),
+    "sddmm_plan_create_opt": (c_int, [c_void_p, c_int32, POINTER(PlanOptions), POINTER(c_void_p)]),
+    "sddmm_plan_create_device_opt": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int32, POINTER(PlanOptions),
+                                             POINTER(c_void_p)]),
+    "sddmm_plan_get_options": (c_int, [c_void_p, POINTER(PlanOptions)]),
     "sddmm_plan_set_values": (c_int, [c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_get_info": (c_int, [c_void_p, POINTER(PlanInfo)]),
     "sddmm_plan_destroy": (None, [c_void_p]),
@@ -84,6 +112,7 @@ SIGNATURES = {
     "sddmm_gpu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_float)]),
     "sddmm_csr_noalloc": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p,
                                   c_void_p, c_void_p]),
+    "sddmm_copy_probe": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "sddmm_device_info": (c_int, [POINTER(c_int), c_char_p, c_int]),
 }
 
@@ -210,10 +239,23 @@ class Coo:
         finally:
             lib().sddmm_tiling_destroy(h)
 
-    def plan(self, K, tile_x=0, tile_y=0, kernel=KERNEL_AUTO):
+    def plan(self, K, tile_x=0, tile_y=0, kernel=KERNEL_AUTO, options=None):
         h = c_void_p()
-        check(lib().sddmm_plan_create(self.h, K, tile_x, tile_y, kernel, byref(h)))
+        if options is not None:
+            check(lib().sddmm_plan_create_opt(self.h, K, byref(options), byref(h)))
+        else:
+            check(lib().sddmm_plan_create(self.h, K, tile_x, tile_y, kernel, byref(h)))
         return Plan(h)
+
+    def cpu(self, K, W, H, n_threads=0):
+        """The SDDMM on the host cores (sddmm_cpu): fp32, sequential sums, no GPU needed."""
+        n_rows, n_cols, nnz, _ = self.info()
+        W = np.ascontiguousarray(W, np.float32)
+        H = np.ascontiguousarray(H, np.float32)
+        assert W.size == n_rows * K and H.size == n_cols * K
+        out = np.empty(nnz, np.float32)
+        check(lib().sddmm_cpu(self.h, K, _np_ptr(W), _np_ptr(H), _np_ptr(out), n_threads))
+        return out
 
     def close(self):
         if self.h:
@@ -237,11 +279,20 @@ class Plan:
 
     @classmethod
     def from_device_csr(cls, n_rows, n_cols, nnz, d_row_ptr, d_col_ind, K, tile_x=0, tile_y=0, kernel=KERNEL_AUTO,
-                        keep=None):
+                        keep=None, options=None):
         h = c_void_p()
-        check(lib().sddmm_plan_create_device(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K, tile_x,
-                                             tile_y, kernel, byref(h)))
+        if options is not None:
+            check(lib().sddmm_plan_create_device_opt(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K,
+                                                     byref(options), byref(h)))
+        else:
+            check(lib().sddmm_plan_create_device(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K, tile_x,
+                                                 tile_y, kernel, byref(h)))
         return cls(h, keep)
+
+    def options(self):
+        o = PlanOptions()
+        check(lib().sddmm_plan_get_options(self.h, byref(o)))
+        return o.as_dict()
 
     def set_values(self, d_val, stream=0):
         check(lib().sddmm_plan_set_values(self.h, c_void_p(d_val), c_void_p(stream or None)))
@@ -301,6 +352,11 @@ def csr_noalloc(n_rows, n_cols, nnz, d_row_ptr, d_col_ind, d_val, K, d_W, d_H, d
     """Plan-free SDDMM over a device CSR that allocates nothing (sddmm_csr_noalloc)."""
     check(lib().sddmm_csr_noalloc(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), c_void_p(d_val or None), K,
                                   c_void_p(d_W), c_void_p(d_H), c_void_p(d_out), c_void_p(stream or None)))
+
+
+def copy_probe(d_src, d_dst, n_bytes, stream=0):
+    """Plain copy kernel of known size (sddmm_copy_probe), the reference HBM counters are scaled by."""
+    check(lib().sddmm_copy_probe(c_void_p(d_src), c_void_p(d_dst), n_bytes, c_void_p(stream or None)))
 
 
 def device_info():

@@ -13,6 +13,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -26,11 +27,21 @@ static void usage()
             "  K              rank of W (rows x K) and H (cols x K)\n"
             "  tile_size_X    columns of S per LDS tile (0 = auto)\n"
             "  tile_size_Y    row-panel height (0 = auto)\n"
-            "options:\n"
             "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
-            "  --kernel NAME  auto | row | lds\n"
+            "                 (the default plan assigns whole column tiles to workgroups and ignores it;\n"
+            "                  it shapes --kernel panel and --kernel lds)\n"
+            "options:\n"
+            "  --ref-order    positionals as the reference binary reads them: K tile_size_Y tile_size_X\n"
+            "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
+            "  --kernel NAME  auto | row | lds | panel | hybrid\n"
             "  --runs N       timed repetitions (default 1; the median is printed)\n"
             "  --save-bin F   write the parsed, sorted matrix to F for fast re-loading\n"
+            "  --check        compare the device result with the CPU path, per nonzero; exit 1 on a mismatch\n"
+            "  --check-against F   compare it, per nonzero, with the nnz raw fp32 values in file F\n"
+            "  --dump-out F   write the result (nnz raw fp32, sorted order) to F\n"
+            "  --cpu-only     run the CPU path only (no GPU needed) and time it\n"
+            "  --cpu-threads N  threads of the CPU path (default: all cores)\n"
+            "  --seed N       srand48 seed of the dense factors (default 0, the reference's)\n"
             "  --json         also print one JSON line with the plan and timing\n");
 }
 
@@ -63,14 +74,23 @@ int main(int argc, char **argv)
     if (*endp || tx < 0) { fprintf(stderr, "sddmm: tile_size_X must be a non-negative integer\n"); return 2; }
     long ty = strtol(argv[4], &endp, 10);
     if (*endp || ty < 0) { fprintf(stderr, "sddmm: tile_size_Y must be a non-negative integer\n"); return 2; }
-    bool transpose = false, json = false;
-    int runs = 1;
+    bool transpose = false, json = false, check = false, cpu_only = false, ref_order = false;
+    int runs = 1, cpu_threads = 0;
+    long seed = 0;
+    std::string check_file, dump_file;
     uint32_t kernel = SDDMM_KERNEL_AUTO;
     std::string save_bin;
     for (int i = 5; i < argc; ++i) {
         std::string a = argv[i];
         if (a == "--transpose") transpose = true;
         else if (a == "--json") json = true;
+        else if (a == "--check") check = true;
+        else if (a == "--cpu-only") cpu_only = true;
+        else if (a == "--ref-order") ref_order = true;
+        else if (a == "--check-against" && i + 1 < argc) check_file = argv[++i];
+        else if (a == "--dump-out" && i + 1 < argc) dump_file = argv[++i];
+        else if (a == "--cpu-threads" && i + 1 < argc) cpu_threads = atoi(argv[++i]);
+        else if (a == "--seed" && i + 1 < argc) seed = atol(argv[++i]);
         else if (a == "--runs" && i + 1 < argc) runs = std::max(1, atoi(argv[++i]));
         else if (a == "--save-bin" && i + 1 < argc) save_bin = argv[++i];
         else if (a == "--kernel" && i + 1 < argc) {
@@ -78,9 +98,12 @@ int main(int argc, char **argv)
             if (k == "auto") kernel = SDDMM_KERNEL_AUTO;
             else if (k == "row") kernel = SDDMM_KERNEL_ROW_GATHER;
             else if (k == "lds") kernel = SDDMM_KERNEL_LDS_TILE;
+            else if (k == "panel") kernel = SDDMM_KERNEL_PANEL;
+            else if (k == "hybrid") kernel = SDDMM_KERNEL_HYBRID;
             else { fprintf(stderr, "sddmm: unknown kernel '%s'\n", k.c_str()); return 2; }
         } else { usage(); return 2; }
     }
+    if (ref_order) std::swap(tx, ty);
 
     auto t0 = std::chrono::steady_clock::now();
     sddmm_coo *S = nullptr;
@@ -98,20 +121,82 @@ int main(int argc, char **argv)
     if (!save_bin.empty()) CHECK(sddmm_write_bin(S, save_bin.c_str()));
     double read_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
 
-    sddmm_plan *plan = nullptr;
-    CHECK(sddmm_plan_create(S, (int32_t)K, (int32_t)tx, (int32_t)ty, kernel, &plan));
-    sddmm_plan_info info;
-    CHECK(sddmm_plan_get_info(plan, &info));
-    printf("\nTilesize: X = %d, tilesize: Y = %d, TB: %d\n", info.tile_size_x, info.tile_size_y, info.block);
-
+    // dense factors: initial() for W and again for H (util.h:75-81; each call reseeds with 0); another
+    // seed draws W, then H, from one drand48 stream
     std::vector<float> W((size_t)n_rows * K), H((size_t)n_cols * K), out((size_t)nnz);
-    CHECK(sddmm_init_reference(W.data(), n_rows, (int32_t)K));
-    CHECK(sddmm_init_reference(H.data(), n_cols, (int32_t)K));
-    std::vector<float> ms((size_t)runs);
-    for (int r = 0; r < runs; ++r) CHECK(sddmm_gpu(plan, W.data(), H.data(), out.data(), &ms[r]));
-    std::sort(ms.begin(), ms.end());
-    float med = ms[ms.size() / 2];
-    printf("\nTime for SDDMM with K = %ld : %g ms\n", K, med);
+    {
+        if (seed == 0) {
+            CHECK(sddmm_init_reference(W.data(), n_rows, (int32_t)K));
+            CHECK(sddmm_init_reference(H.data(), n_cols, (int32_t)K));
+        } else {
+            srand48(seed);
+            for (auto &x : W) x = (float)(0.1 * drand48());
+            for (auto &x : H) x = (float)(0.1 * drand48());
+        }
+    }
+    std::vector<float> cpu;
+    double cpu_ms = 0;
+    if (check || cpu_only) {
+        cpu.resize((size_t)nnz);
+        auto c0 = std::chrono::steady_clock::now();
+        CHECK(sddmm_cpu(S, (int32_t)K, W.data(), H.data(), cpu.data(), cpu_threads));
+        cpu_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - c0).count();
+        printf("\nTime for CPU SDDMM with K = %ld : %g ms\n", K, cpu_ms);
+    }
+
+    sddmm_plan *plan = nullptr;
+    sddmm_plan_info info;
+    memset(&info, 0, sizeof info);
+    float med = 0.f;
+    if (cpu_only) {
+        out = cpu;
+        printf("\nTilesize: X = %ld, tilesize: Y = %ld, TB: 0\n", tx, ty);
+    } else {
+        CHECK(sddmm_plan_create(S, (int32_t)K, (int32_t)tx, (int32_t)ty, kernel, &plan));
+        CHECK(sddmm_plan_get_info(plan, &info));
+        printf("\nTilesize: X = %d, tilesize: Y = %d, TB: %d\n", info.tile_size_x, info.tile_size_y, info.block);
+        std::vector<float> ms((size_t)runs);
+        for (int r = 0; r < runs; ++r) CHECK(sddmm_gpu(plan, W.data(), H.data(), out.data(), &ms[r]));
+        std::sort(ms.begin(), ms.end());
+        med = ms[ms.size() / 2];
+        printf("\nTime for SDDMM with K = %ld : %g ms\n", K, med);
+    }
+    if (!dump_file.empty()) {
+        FILE *f = fopen(dump_file.c_str(), "wb");
+        if (!f || fwrite(out.data(), 4, out.size(), f) != out.size()) {
+            fprintf(stderr, "sddmm: cannot write %s\n", dump_file.c_str());
+            return 12;
+        }
+        fclose(f);
+    }
+    // Per-nonzero comparison.  The reference counts |gpu - cpu| > 1e-6 (sddmm.cu:133-141); with factors of
+    // other magnitudes an absolute bound says little, so the count here uses the relative bound
+    // 1e-5*sqrt(K)*|expected| with an absolute floor of 1e-6, and both counts are printed.
+    long long diff_tot = -1, diff_abs = -1;
+    double max_rel = 0;
+    if (!check_file.empty()) {
+        cpu.resize((size_t)nnz);
+        FILE *f = fopen(check_file.c_str(), "rb");
+        if (!f || fread(cpu.data(), 4, cpu.size(), f) != cpu.size() || fgetc(f) != EOF) {
+            fprintf(stderr, "sddmm: %s does not hold exactly %lld fp32 values\n", check_file.c_str(), (long long)nnz);
+            return 12;
+        }
+        fclose(f);
+    }
+    if ((check && !cpu_only) || !check_file.empty()) {
+        diff_tot = 0; diff_abs = 0;
+        const double tol = 1e-5 * std::sqrt((double)K);
+        for (int64_t i = 0; i < nnz; ++i) {
+            const double e = cpu[(size_t)i], d = std::fabs((double)out[(size_t)i] - e);
+            if (!(d <= tol * std::fabs(e) + 1e-6)) {
+                if (diff_tot < 5) printf("expected/got diff %lld:  %g %g %g\n", (long long)i, e, (double)out[(size_t)i], d);
+                ++diff_tot;
+            }
+            if (!(d <= 1e-6)) ++diff_abs;
+            if (e != 0) max_rel = std::max(max_rel, d / std::fabs(e));
+        }
+        printf("\ndiff values in CPU and GPU: %lld (|diff| > 1e-6: %lld, max relative %.3g)\n", diff_tot, diff_abs, max_rel);
+    }
     double sum = 0;
     for (float v : out) sum += v;
     if (json) {
@@ -120,12 +205,12 @@ int main(int argc, char **argv)
         printf("{\"rows\": %lld, \"cols\": %lld, \"nnz\": %lld, \"K\": %ld, \"tile_size_x\": %d, \"tile_size_y\": %d, "
                "\"kernel\": %d, \"lanes_per_nnz\": %d, \"lds_bytes\": %d, \"grid\": %d, \"block\": %d, "
                "\"n_col_tiles\": %d, \"read_ms\": %.3f, \"plan_ms\": %.3f, \"kernel_ms\": %.6f, \"gflops\": %.3f, "
-               "\"alg_gbps\": %.3f, \"checksum\": %.9g}\n",
+               "\"alg_gbps\": %.3f, \"cpu_ms\": %.3f, \"mismatches\": %lld, \"max_rel\": %.4g, \"checksum\": %.9g}\n",
                (long long)n_rows, (long long)n_cols, (long long)nnz, K, info.tile_size_x, info.tile_size_y, info.kernel,
                info.lanes_per_nnz, info.lds_bytes, info.grid, info.block, info.n_col_tiles, read_ms, info.plan_ms,
-               (double)med, gflops, med > 0 ? balg / (med * 1e6) : 0.0, sum);
+               (double)med, gflops, med > 0 ? balg / (med * 1e6) : 0.0, cpu_ms, diff_tot, max_rel, sum);
     }
     sddmm_plan_destroy(plan);
     sddmm_coo_destroy(S);
-    return 0;
+    return diff_tot > 0 ? 1 : 0;
 }

@@ -2,9 +2,12 @@
 // sort, transposing sort, CSR / compressed-CSR pointers, reference-style dense
 // factor initialisation.  Plain C++17 + std::thread; no GPU calls here.
 #include "internal.hpp"
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <mutex>
 #include <numeric>
 #include <string>
 
@@ -56,13 +59,55 @@ void parallel_ranges(int64_t n, int64_t grain, const std::function<void(int64_t,
         f(0, n, 0);
         return;
     }
+    // an exception in a worker (an allocation that fails) is carried to the caller
+    std::exception_ptr err;
+    std::mutex err_mu;
     std::vector<std::thread> th;
     th.reserve(nt);
     for (int t = 0; t < nt; ++t) {
         int64_t b = n * t / nt, e = n * (t + 1) / nt;
-        th.emplace_back([&f, b, e, t] { f(b, e, t); });
+        th.emplace_back([&f, &err, &err_mu, b, e, t] {
+            try {
+                f(b, e, t);
+            } catch (...) {
+                std::lock_guard<std::mutex> g(err_mu);
+                if (!err) err = std::current_exception();
+            }
+        });
     }
     for (auto &x : th) x.join();
+    if (err) std::rethrow_exception(err);
+}
+
+void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t, int64_t, int)> &f)
+{
+    chunk = std::max<int64_t>(chunk, 1);
+    const int nt = (int)std::max<int64_t>(1, std::min<int64_t>(hw_threads(), (n + chunk - 1) / chunk));
+    if (nt == 1) {
+        if (n > 0) f(0, n, 0);
+        return;
+    }
+    std::atomic<int64_t> next{0};
+    std::exception_ptr err;
+    std::mutex err_mu;
+    std::vector<std::thread> th;
+    th.reserve(nt);
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([&, t] {
+            try {
+                for (;;) {
+                    const int64_t b = next.fetch_add(chunk);
+                    if (b >= n) break;
+                    f(b, std::min(n, b + chunk), t);
+                }
+            } catch (...) {
+                next.store(n);  // the others stop at their next chunk
+                std::lock_guard<std::mutex> g(err_mu);
+                if (!err) err = std::current_exception();
+            }
+        });
+    for (auto &x : th) x.join();
+    if (err) std::rethrow_exception(err);
 }
 
 bool check_sorted(const sddmm_coo &S)
@@ -166,11 +211,11 @@ int sddmm_coo_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t 
         S->cols.assign(cols, cols + nnz);
         if (vals) S->vals.assign(vals, vals + nnz);
         else S->vals.assign((size_t)nnz, 1.0f);
-    } catch (const std::bad_alloc &) {
+        S->sorted = check_sorted(*S) ? 1 : 0;
+    } catch (const std::exception &e) {
         delete S;
-        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_create: out of memory");
+        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_create: %s", e.what());
     }
-    S->sorted = check_sorted(*S) ? 1 : 0;
     *out = S;
     return SDDMM_OK;
 }
@@ -183,10 +228,7 @@ int sddmm_coo_info(const sddmm_coo *S, int64_t *n_rows, int64_t *n_cols, int64_t
     if (n_rows) *n_rows = S->n_rows;
     if (n_cols) *n_cols = S->n_cols;
     if (nnz) *nnz = S->nnz;
-    if (sorted) {
-        if (S->sorted < 0) const_cast<sddmm_coo *>(S)->sorted = check_sorted(*S) ? 1 : 0;
-        *sorted = S->sorted;
-    }
+    if (sorted) *sorted = S->sorted == 1;
     return SDDMM_OK;
 }
 
@@ -202,12 +244,11 @@ int sddmm_coo_arrays(const sddmm_coo *S, const int32_t **rows, const int32_t **c
 int sddmm_coo_sort_rows(sddmm_coo *S)
 {
     if (!S) return fail(SDDMM_ERR_ARG, "sddmm_coo_sort_rows: S is NULL");
-    if (S->sorted < 0) S->sorted = check_sorted(*S) ? 1 : 0;
     if (S->sorted == 1) return SDDMM_OK;
     try {
         sort_row_col(*S);
-    } catch (const std::bad_alloc &) {
-        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_sort_rows: out of memory");
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_sort_rows: %s", e.what());
     }
     return SDDMM_OK;
 }
@@ -217,12 +258,13 @@ int sddmm_coo_transpose_sort(sddmm_coo *S)
     if (!S) return fail(SDDMM_ERR_ARG, "sddmm_coo_transpose_sort: S is NULL");
     S->rows.swap(S->cols);
     std::swap(S->n_rows, S->n_cols);
-    S->sorted = check_sorted(*S) ? 1 : 0;
-    if (S->sorted == 1) return SDDMM_OK;
+    S->sorted = 0;
     try {
+        S->sorted = check_sorted(*S) ? 1 : 0;
+        if (S->sorted == 1) return SDDMM_OK;
         sort_row_col(*S);
-    } catch (const std::bad_alloc &) {
-        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_transpose_sort: out of memory");
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_transpose_sort: %s", e.what());
     }
     return SDDMM_OK;
 }
@@ -230,7 +272,6 @@ int sddmm_coo_transpose_sort(sddmm_coo *S)
 static int need_sorted(const sddmm_coo *S, const char *who)
 {
     if (!S) return fail(SDDMM_ERR_ARG, "%s: S is NULL", who);
-    if (S->sorted < 0) const_cast<sddmm_coo *>(S)->sorted = check_sorted(*S) ? 1 : 0;
     if (S->sorted != 1) return fail(SDDMM_ERR_UNSORTED, "%s: matrix is not (row, col)-sorted; call sddmm_coo_sort_rows", who);
     return SDDMM_OK;
 }
@@ -239,9 +280,13 @@ int sddmm_coo_row_ptr(const sddmm_coo *S, int32_t *row_ptr)
 {
     if (int rc = need_sorted(S, "sddmm_coo_row_ptr")) return rc;
     if (!row_ptr) return fail(SDDMM_ERR_ARG, "sddmm_coo_row_ptr: row_ptr is NULL");
-    std::vector<int32_t> rp;
-    build_row_ptr(*S, rp);
-    memcpy(row_ptr, rp.data(), rp.size() * sizeof(int32_t));
+    try {
+        std::vector<int32_t> rp;
+        build_row_ptr(*S, rp);
+        memcpy(row_ptr, rp.data(), rp.size() * sizeof(int32_t));
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_row_ptr: %s", e.what());
+    }
     return SDDMM_OK;
 }
 
@@ -250,7 +295,11 @@ int sddmm_coo_compress_rows(const sddmm_coo *S, int32_t *row_ptr, int32_t *row_h
     if (int rc = need_sorted(S, "sddmm_coo_compress_rows")) return rc;
     if (!row_ptr || !row_holder) return fail(SDDMM_ERR_ARG, "sddmm_coo_compress_rows: NULL output");
     std::vector<int32_t> rp;
-    build_row_ptr(*S, rp);
+    try {
+        build_row_ptr(*S, rp);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_coo_compress_rows: %s", e.what());
+    }
     int64_t h = 0;
     row_ptr[0] = 0;
     for (int64_t r = 0; r < S->n_rows; ++r) {
@@ -260,6 +309,47 @@ int sddmm_coo_compress_rows(const sddmm_coo *S, int32_t *row_ptr, int32_t *row_h
         }
     }
     if (n_nonempty) *n_nonempty = h;
+    return SDDMM_OK;
+}
+
+// The product's own CPU path: rows dealt to threads in chunks, every nonzero a
+// sequential fp32 sum over K (t ascending), scaled by the value last -- the
+// arithmetic of sddmm_CPU_CSR, HiPC18/src/sddmm.cu:153-177.
+int sddmm_cpu(const sddmm_coo *S, int32_t K, const float *W, const float *H, float *out, int32_t n_threads)
+{
+    if (int rc = need_sorted(S, "sddmm_cpu")) return rc;
+    if (K < 1) return fail(SDDMM_ERR_ARG, "sddmm_cpu: K must be >= 1 (got %d)", K);
+    if (S->nnz > 0 && (!W || !H || !out)) return fail(SDDMM_ERR_ARG, "sddmm_cpu: NULL argument");
+    if (S->nnz == 0) return SDDMM_OK;
+    try {
+        const int64_t nnz = S->nnz;
+        const int32_t *rows = S->rows.data(), *cols = S->cols.data();
+        const float *vals = S->vals.data();
+        int nt = n_threads > 0 ? std::min<int>(n_threads, 256) : hw_threads();
+        const int64_t chunk = std::max<int64_t>(1024, nnz / (64 * (int64_t)nt));
+        nt = (int)std::max<int64_t>(1, std::min<int64_t>(nt, (nnz + chunk - 1) / chunk));
+        std::atomic<int64_t> next{0};
+        auto work = [&] {
+            for (;;) {
+                const int64_t b = next.fetch_add(chunk);
+                if (b >= nnz) break;
+                const int64_t e = std::min(nnz, b + chunk);
+                for (int64_t p = b; p < e; ++p) {
+                    const float *w = W + (int64_t)rows[p] * K, *h = H + (int64_t)cols[p] * K;
+                    float sm = 0.f;
+                    for (int32_t t = 0; t < K; ++t) sm += w[t] * h[t];
+                    out[p] = sm * vals[p];
+                }
+            }
+        };
+        std::vector<std::thread> th;
+        th.reserve((size_t)nt);
+        for (int t = 1; t < nt; ++t) th.emplace_back(work);
+        work();
+        for (auto &x : th) x.join();
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_cpu: %s", e.what());
+    }
     return SDDMM_OK;
 }
 

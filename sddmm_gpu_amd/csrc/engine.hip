@@ -43,6 +43,8 @@ struct Launch {
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
+    DenseFn dfn = nullptr;       // dense-block kernel; null: not a dense launch
+    DenseArgs da{};
     float *sval = nullptr;        // the plan's values in stream order (launches that walk a permuted stream)
     const int32_t *perm = nullptr;  // stream position -> sorted position of that launch (null: identity)
     int32_t grid = 0, block = 0, lds = 0, k_slice = 0;
@@ -57,6 +59,7 @@ struct sddmm_plan {
     const int32_t *d_row_ptr = nullptr, *d_col = nullptr;
     float *d_val = nullptr;
     int32_t requested_kernel = 0;
+    sddmm_plan_options options{};  // what the plan was built with, environment overrides applied
     ~sddmm_plan()
     {
         for (void *p : owned) (void)hipFree(p);
@@ -137,10 +140,17 @@ struct Ctx {
     sddmm_plan *P;
     int64_t n_rows, n_cols, nnz;
     const int32_t *row_ptr, *col_ind;  // host CSR
-    const float *vals;                 // host values or null
+    const float *vals;                 // host values (indexed by position in the original S) or null
     int32_t K;
     int cus;
     int64_t dev_bytes = 0;
+    // The CSR above may be what is left of S after the dense blocks were cut out; orig then maps
+    // its positions to positions in the original S (null: the CSR is S itself).  Streams record
+    // original positions: that is where outputs go and where values come from.
+    const int32_t *orig = nullptr;
+    sddmm_plan_options opt{};  // the caller's options with the environment overrides applied
+    int32_t pos(int64_t p) const { return orig ? orig[p] : (int32_t)p; }
+    float value(int64_t p) const { return vals[orig ? orig[p] : p]; }
 
     template <class T>
     int up(T **dst, const std::vector<T> &src)
@@ -171,6 +181,35 @@ int64_t env_i64(const char *name, int64_t dflt)
     return (end && *end == 0) ? (int64_t)v : dflt;
 }
 
+void default_options(sddmm_plan_options &o)
+{
+    o.kernel = SDDMM_KERNEL_AUTO;
+    o.tile_size_x = 0; o.tile_size_y = 0;
+    o.k_slice = -1; o.tile_lanes = -1; o.tile_waves = -1; o.tile_assign = -1; o.tile_few_blocks = -1;
+    o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.gather_lanes = -1; o.gather_padded = -1;
+    o.gather_sink = -1; o.row_padded = -1; o.unpadded_tile = -1; o.dense_blocks = -1; o.dense_permille = -1;
+    o.dense_rb_group = -1; o.ignore_env = 0;
+    o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
+}
+
+// The environment as an override layer over the caller's options.
+void apply_env_overrides(sddmm_plan_options &o)
+{
+    if (o.ignore_env) return;
+    auto i32 = [](const char *name, int32_t &v) { v = (int32_t)env_i64(name, v); };
+    auto i64 = [](const char *name, int64_t &v) { v = env_i64(name, v); };
+    i32("SDDMM_KERNEL", o.kernel); i32("SDDMM_TILE_X", o.tile_size_x); i32("SDDMM_TILE_Y", o.tile_size_y);
+    i32("SDDMM_TILE_KSLICE", o.k_slice); i32("SDDMM_TILE_G", o.tile_lanes); i32("SDDMM_TILE_WAVES", o.tile_waves);
+    i32("SDDMM_TILE_ASSIGN", o.tile_assign); i32("SDDMM_TILE_FEW_BLOCKS", o.tile_few_blocks);
+    i32("SDDMM_TILE_SHORT", o.tile_short_batches); i32("SDDMM_TILE_DEAL", o.tile_deal); i32("SDDMM_TILE_RUNS", o.tile_runs);
+    i32("SDDMM_GATHER_G", o.gather_lanes); i32("SDDMM_GATHER_PADDED", o.gather_padded); i32("SDDMM_GATHER_SINK", o.gather_sink);
+    i32("SDDMM_ROW_PADDED", o.row_padded); i32("SDDMM_UNPADDED_TILE", o.unpadded_tile); i32("SDDMM_DENSE", o.dense_blocks);
+    i32("SDDMM_DENSE_PERMILLE", o.dense_permille); i32("SDDMM_DENSE_RB_GROUP", o.dense_rb_group);
+    i64("SDDMM_DENSE_MIN_NNZ", o.dense_min_nnz); i64("SDDMM_PANEL_BYTES", o.panel_bytes);
+    i64("SDDMM_SHORT_ROW_MAX", o.short_row_max); i64("SDDMM_STAGE_FACTOR", o.stage_factor);
+    i64("SDDMM_SPLIT_MIN_NNZ", o.split_min_nnz);
+}
+
 int64_t list_nnz(const Ctx &c, const std::vector<int32_t> &rows)
 {
     int64_t n = 0;
@@ -185,6 +224,7 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
     Launch L;
     L.kind = SDDMM_KERNEL_ROW_GATHER;
     L.rows = (int64_t)rows.size();
+    if (c.orig) all_rows = false;  // positions of the remainder are not positions of S
     const int64_t n = all_rows ? c.nnz : list_nnz(c, rows);
     L.nnz = n;
     if (n == 0) return SDDMM_OK;
@@ -203,7 +243,7 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
         parallel_ranges((int64_t)rows.size(), 1 << 10, [&](int64_t b, int64_t e, int) {
             for (int64_t i = b; i < e; ++i) {
                 int64_t d = i ? seg_end[i - 1] : 0;
-                for (int32_t p = c.row_ptr[rows[i]]; p < c.row_ptr[rows[i] + 1]; ++p) perm[d++] = p;
+                for (int32_t p = c.row_ptr[rows[i]]; p < c.row_ptr[rows[i] + 1]; ++p) perm[d++] = c.pos(p);
             }
         });
     }
@@ -284,9 +324,13 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     if (c.vals) {
         sval.resize((size_t)n);
         parallel_ranges(n, 1 << 16, [&](int64_t b, int64_t e, int) {
-            for (int64_t i = b; i < e; ++i) sval[i] = c.vals[T.tiled_ind[i]];
+            for (int64_t i = b; i < e; ++i) sval[i] = c.value(T.tiled_ind[i]);
         });
     }
+    if (c.orig)
+        parallel_ranges(n, 1 << 16, [&](int64_t b, int64_t e, int) {
+            for (int64_t i = b; i < e; ++i) T.tiled_ind[i] = c.orig[T.tiled_ind[i]];
+        });
     KArgs &a = L.ka;
     int32_t *d_perm = nullptr, *d_seg_row = nullptr, *d_bseg = nullptr, *d_scol = nullptr;
     uint64_t *d_bmask = nullptr;
@@ -301,7 +345,7 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     if (int rc = c.up(&d_sval, sval)) return rc;
     a.perm = d_perm; a.seg_row = d_seg_row; a.items = d_items; a.batch_seg = d_bseg; a.batch_mask = d_bmask;
     a.scol = d_scol;
-    L.sval = d_sval; L.perm = d_perm;
+    L.sval = d_sval; L.perm = d_perm; L.positions = n;
     a.n_items = (int32_t)items.size();
     a.nnz = (int32_t)n; a.K = c.K; a.tile_x = x; a.n_cols = (int32_t)c.n_cols;
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)items.size()));
@@ -333,7 +377,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
     // 12 waves per workgroup measured 2-5 % faster than 16 on slices of 64 and 128, slower on 32
-    int nwaves = gather ? 4 : (int)env_i64("SDDMM_TILE_WAVES", ks >= 64 ? 12 : 16);
+    int nwaves = gather ? 4 : (int)(c.opt.tile_waves > 0 ? c.opt.tile_waves : (ks >= 64 ? 12 : 16));
     if (!gather && nwaves != 12) nwaves = 16;
     L.tfn = tv.G ? tile_kernel(tv, 0, gather, false, nwaves) : nullptr;
     if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
@@ -349,7 +393,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // tile is staged once) and one of `shares` row blocks that are the same for all
     // tiles, so the workgroups of different tiles read the same W rows at about the same
     // time and share them in L2.  The tile count is raised to a divisor of the CU count.
-    const int assign = (int)env_i64("SDDMM_TILE_ASSIGN", 2);
+    const int assign = (int)(c.opt.tile_assign >= 0 ? c.opt.tile_assign : 2);
     bool grid2d = !gather && assign != 0;
     int shares = 1;
     // xcd_local: workgroup b runs on die b % 8 (round-robin dispatch), each die has its
@@ -372,7 +416,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 // twice a tile's bytes in index data -- the assignment with the fewest row blocks wins)
                 const bool staging_dominates = 8.0 * (double)nt * x * ks * 4 > 2.0 * 12.5 * (double)L.nnz;
                 if (assign == 2 && c.cus % 8 == 0 && nt == n2 && (n2 % per_die == 0 || per_die % n2 == 0) &&
-                    !(staging_dominates && env_i64("SDDMM_TILE_FEW_BLOCKS", 1) != 0)) {
+                    !(staging_dominates && c.opt.tile_few_blocks != 0)) {
                     xcd_local = true;
                     xcd_steps = (int)std::max<int64_t>(1, n2 / per_die);
                     shares = 8 * (int)std::max<int64_t>(1, per_die / n2);
@@ -386,10 +430,10 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // Short batches (see tile_variant_shorts): the last chunk of a (row, tile) run that holds at
     // most G/2 nonzeros is kept apart from the full chunks, and eight such chunks make a batch of
     // their own, which the kernel runs in half the steps.
-    const bool shorts = grid2d && tile_variant_shorts(tv.G, tv.KPL, gather) && env_i64("SDDMM_TILE_SHORT", 1) != 0;
+    const bool shorts = grid2d && tile_variant_shorts(tv.G, tv.KPL, gather) && c.opt.tile_short_batches != 0;
     // gather form: padding positions are flagged and their results go to a scratch line
-    const bool flag_padding = gather && env_i64("SDDMM_GATHER_SINK", 1) != 0;
-    const bool deal_tiles = env_i64("SDDMM_TILE_DEAL", 1) != 0;
+    const bool flag_padding = gather && c.opt.gather_sink != 0;
+    const bool deal_tiles = c.opt.tile_deal != 0;
     std::vector<uint32_t> btype;
     std::vector<WorkItem> items;
     // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
@@ -484,9 +528,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                         int64_t d = d0;
                         for (int i = 0; i < ch.cnt; ++i, ++d) {
                             const int32_t p = T.tiled_ind[b + ch.e0 + i];
-                            perm[(size_t)d] = p;
+                            perm[(size_t)d] = c.pos(p);
                             scol[(size_t)d] = (c.col_ind[p] - tile_base) * row_bytes;
-                            if (c.vals) sval[(size_t)d] = c.vals[p];
+                            if (c.vals) sval[(size_t)d] = c.value(p);
                         }
                         for (; d < d0 + span; ++d) {  // padding repeats the chunk's last nonzero
                             perm[(size_t)d] = perm[(size_t)d - 1]; scol[(size_t)d] = scol[(size_t)d - 1];
@@ -561,10 +605,10 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                 int64_t d = poff[s];
                 for (int64_t i = 0; i < len; ++i, ++d) {
                     const int32_t p = T.tiled_ind[b + i];
-                    perm[d] = p;
+                    perm[d] = c.pos(p);
                     // byte offset of the H row inside the LDS tile (gather form: index of its first float4 in H)
                     scol[d] = gather ? (int32_t)((uint32_t)c.col_ind[p] * k4) : (c.col_ind[p] - tile_base) * row_bytes;
-                    if (c.vals) sval[d] = c.vals[p];
+                    if (c.vals) sval[d] = c.value(p);
                 }
                 // padding repeats the run's last nonzero: the kernel stores every position
                 // without a test, and a repeat stores the same result at the same place
@@ -638,7 +682,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                         items.push_back(item_of(sh, j));
                     }
             } else if (shares == 1 && c.cus % 8 == 0 && (int64_t)tiles_ne.size() > c.cus &&
-                       env_i64("SDDMM_TILE_RUNS", 1) != 0) {
+                       c.opt.tile_runs != 0) {
                 // More tiles than workgroups (a wide matrix; one item per tile, all rows).  Neighbouring
                 // tiles of a banded matrix share most of their rows: each turn gives a run of
                 // consecutive tiles to the workgroups of one die (workgroup b runs on die b % 8), so
@@ -678,6 +722,8 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // VALU issue and the 6 extra instructions per batch cost more than the bytes save.  perm
     // stays on the device for sddmm_plan_set_values only.
     const bool compact = !gather && ks / 4 <= 16;
+    // (the compact form needs a group's nonzeros at consecutive positions of S: not so in a remainder)
+    if (compact && c.orig) return fail(SDDMM_ERR_ARG, "plan: compact tile stream over a remainder matrix");
     if (compact) {
         const int64_t ng = np / G;
         std::vector<uint16_t> scol16((size_t)np + kStreamSlack, 0);
@@ -739,6 +785,80 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     }
     c.P->info.padded_positions += np;
     L.positions = np; L.tile_g = G;
+    c.P->launches.push_back(L);
+    return SDDMM_OK;
+}
+
+// Dense-block launch: the blocks found by find_dense_blocks, one workgroup per block at a time.
+int add_dense(Ctx &c, const DenseBlocks &D, const float *vals_all)
+{
+    Launch L;
+    L.kind = SDDMM_KERNEL_DENSE_BLOCK;
+    L.dfn = dense_kernel();
+    L.nnz = D.n_dense;
+    const int64_t n_tiles = (int64_t)D.tile_rb.size();
+    // Schedule: workgroup b runs on die b % 8 (each die has its own L2) and takes slots b, b + grid, ...
+    // The blocks are ordered by (group of 8 row blocks, column group, row block) and cut into 8
+    // consecutive parts, one per die: the workgroups of a die then work on a few row blocks times a
+    // few neighbouring column groups at a time, so the W rows of those row blocks stay in that L2
+    // for the whole sweep over the columns and an H row is fetched once for the 8 row blocks that
+    // use it (row blocks of similar length have about the same dense columns).
+    const int rb_group = (int)std::max<int64_t>(1, (c.opt.dense_rb_group > 0 ? c.opt.dense_rb_group : 8));
+    std::vector<int32_t> order((size_t)n_tiles), cg((size_t)n_tiles);
+    for (int64_t k = 0; k < n_tiles; ++k) {
+        order[(size_t)k] = (int32_t)k;
+        cg[(size_t)k] = (k > 0 && D.tile_rb[(size_t)k] == D.tile_rb[(size_t)k - 1]) ? cg[(size_t)k - 1] + 1 : 0;
+    }
+    std::sort(order.begin(), order.end(), [&](int32_t x, int32_t y) {
+        const int32_t gx = D.tile_rb[(size_t)x] / rb_group, gy = D.tile_rb[(size_t)y] / rb_group;
+        if (gx != gy) return gx < gy;
+        if (cg[(size_t)x] != cg[(size_t)y]) return cg[(size_t)x] < cg[(size_t)y];
+        return x < y;
+    });
+    const int grid = (int)std::max<int64_t>(8, std::min<int64_t>(2 * (int64_t)c.cus, (n_tiles + 7) / 8 * 8)) / 8 * 8;
+    const int per_die = grid / 8;
+    const int64_t part = (n_tiles + 7) / 8;
+    const int64_t turns = (part + per_die - 1) / per_die;
+    const int64_t n_slots = turns * grid;
+    const int T = D.tile;
+    std::vector<int32_t> slot_rows((size_t)(n_slots * T), 0), slot_cols((size_t)(n_slots * T), 0);
+    std::vector<int2> slot_range((size_t)n_slots, make_int2(0, 0));
+    for (int die = 0; die < 8; ++die)
+        for (int64_t j = 0; j < part; ++j) {
+            if (die * part + j >= n_tiles) break;
+            const int64_t tile = order[(size_t)(die * part + j)];
+            const int64_t slot = (j / per_die) * grid + (j % per_die) * 8 + die;
+            std::copy(D.row_ids.begin() + (size_t)D.tile_rb[(size_t)tile] * T, D.row_ids.begin() + ((size_t)D.tile_rb[(size_t)tile] + 1) * T,
+                      slot_rows.begin() + (size_t)(slot * T));
+            std::copy(D.col_ids.begin() + (size_t)tile * T, D.col_ids.begin() + ((size_t)tile + 1) * T, slot_cols.begin() + (size_t)(slot * T));
+            slot_range[(size_t)slot] = make_int2(D.tile_ptr[(size_t)tile], D.tile_ptr[(size_t)tile + 1]);
+        }
+    std::vector<float> nz_val;
+    if (vals_all) {
+        nz_val.resize((size_t)D.n_dense);
+        parallel_ranges(D.n_dense, 1 << 16, [&](int64_t b, int64_t e, int) {
+            for (int64_t i = b; i < e; ++i) nz_val[(size_t)i] = vals_all[D.nz_p[(size_t)i]];
+        });
+    }
+    int32_t *d_rows = nullptr, *d_cols = nullptr, *d_p = nullptr;
+    int2 *d_range = nullptr;
+    uint16_t *d_rc = nullptr;
+    float *d_v = nullptr;
+    if (int rc = c.up(&d_rows, slot_rows)) return rc;
+    if (int rc = c.up(&d_cols, slot_cols)) return rc;
+    if (int rc = c.up(&d_range, slot_range)) return rc;
+    if (int rc = c.up(&d_p, D.nz_p)) return rc;
+    if (int rc = c.up(&d_rc, D.nz_rc)) return rc;
+    if (int rc = c.up(&d_v, nz_val)) return rc;
+    DenseArgs &a = L.da;
+    a.slot_rows = d_rows; a.slot_cols = d_cols; a.slot_range = d_range;
+    a.nz_p = d_p; a.nz_rc = d_rc;
+    a.n_slots = (int32_t)n_slots; a.K = c.K;
+    L.sval = d_v; L.perm = d_p; L.positions = D.n_dense;
+    L.grid = grid; L.block = 256; L.lds = 0; L.k_slice = c.K;
+    L.rows = (int64_t)D.row_ids.size();
+    c.P->info.dense_nnz = D.n_dense;
+    c.P->info.dense_blocks = n_tiles;
     c.P->launches.push_back(L);
     return SDDMM_OK;
 }
@@ -819,10 +939,14 @@ int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, 
 
 // Common plan builder from host CSR arrays.  d_*_borrowed != null: the device
 // already holds that array.
-int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr, const int32_t *col_ind,
+int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr_all, const int32_t *col_ind_all,
               const float *vals, const int32_t *d_row_ptr_borrowed, const int32_t *d_col_borrowed, int32_t K,
-              int32_t tile_x, int32_t tile_y, uint32_t flags, sddmm_plan **out)
+              const sddmm_plan_options &opt_in, sddmm_plan **out)
 {
+    sddmm_plan_options opt = opt_in;
+    apply_env_overrides(opt);
+    if (opt.tile_lanes < 0) opt.tile_lanes = 0;  // (0 is "choose" for the variant pickers)
+    const int32_t tile_x = opt.tile_size_x, tile_y = opt.tile_size_y;
     auto t0 = std::chrono::steady_clock::now();
     if (K < 1) return fail(SDDMM_ERR_ARG, "plan: K must be >= 1 (got %d)", K);
     if (tile_x < 0 || tile_y < 0) return fail(SDDMM_ERR_ARG, "plan: tile sizes must be >= 0");
@@ -831,7 +955,8 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     if ((n_rows * (int64_t)K) >= (int64_t)1 << 40 || (n_cols * (int64_t)K) >= (int64_t)1 << 40)
         return fail(SDDMM_ERR_RANGE, "plan: dense factor too large");
     if (int rc = device_ok()) return rc;
-    int want = (int)(flags & 0xff);
+    int want = opt.kernel;
+    if (want < 0) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
     if (want > SDDMM_KERNEL_HYBRID) return fail(SDDMM_ERR_ARG, "plan: unknown kernel id %d", want);
 
     sddmm_plan *P = new (std::nothrow) sddmm_plan;
@@ -839,12 +964,17 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     struct Guard { sddmm_plan *p; ~Guard() { delete p; } } guard{P};
     sddmm_plan_info &I = P->info;
     I.n_rows = n_rows; I.n_cols = n_cols; I.nnz = nnz; I.K = K; I.k_slice = K;
-    count_touched(n_rows, n_cols, nnz, row_ptr, col_ind, &I.rows_touched, &I.cols_touched);
+    count_touched(n_rows, n_cols, nnz, row_ptr_all, col_ind_all, &I.rows_touched, &I.cols_touched);
     P->requested_kernel = want;
+    // what the gathering kernels work on: S itself, or what is left of it once the dense blocks are cut out
+    const int32_t *row_ptr = row_ptr_all, *col_ind = col_ind_all;
+    int64_t nnz_part = nnz;
 
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, 0));
-    Ctx c{P, n_rows, n_cols, nnz, row_ptr, col_ind, vals, K, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
+    Ctx c{P, n_rows, n_cols, nnz, row_ptr_all, col_ind_all, vals, K, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
+    c.opt = opt;
+    P->options = opt;
 
     P->d_row_ptr = d_row_ptr_borrowed;
     if (d_col_borrowed) {
@@ -853,7 +983,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         int32_t *d = nullptr;
         HIP_TRY(hipMalloc((void **)&d, (size_t)nnz * 4));
         P->owned.push_back(d);
-        HIP_TRY(hipMemcpy(d, col_ind, (size_t)nnz * 4, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(d, col_ind_all, (size_t)nnz * 4, hipMemcpyHostToDevice));
         c.dev_bytes += nnz * 4;
         P->d_col = d;
     }
@@ -863,12 +993,6 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         HIP_TRY(hipMemcpy(P->d_val, vals, (size_t)nnz * 4, hipMemcpyHostToDevice));
         c.dev_bytes += nnz * 4;
     }
-
-    // non-empty rows, ascending
-    std::vector<int32_t> ne;
-    ne.reserve((size_t)I.rows_touched);
-    for (int64_t r = 0; r < n_rows; ++r)
-        if (row_ptr[r + 1] > row_ptr[r]) ne.push_back((int32_t)r);
 
     const bool have_vec = (K % 4 == 0) && pick_variant(K, true).G != 0;
     const int64_t row_bytes = (int64_t)K * 4;
@@ -881,15 +1005,12 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     else if (K > 128 && K % 128 == 0) kt = 128;
     else if (K > 128 && K % 64 == 0) kt = 64;
     else if (pick_tile_variant(K, 0).G) kt = K;
-    {
-        const int64_t o = env_i64("SDDMM_TILE_KSLICE", 0);
-        if (o > 0 && K % o == 0 && pick_tile_variant((int)o, 0).G) kt = (int)o;
-    }
+    if (opt.k_slice > 0 && K % opt.k_slice == 0 && pick_tile_variant(opt.k_slice, 0).G) kt = opt.k_slice;
     const int32_t fit_t = kt ? kLdsMaxBytes / (kt * 4) : 0;  // H rows per LDS tile of the tile kernel
 
     // row-panel height of the tile kernel's stream: the panel's W slice (y rows of kt floats)
     // should stay L2-resident while the workgroups sweep the panel's column tiles
-    int32_t y_panel = tile_y > 0 ? tile_y : (kt ? (int32_t)std::max<int64_t>(256, env_i64("SDDMM_PANEL_BYTES", 2 << 20) / (kt * 4)) : 1);
+    int32_t y_panel = tile_y > 0 ? tile_y : (kt ? (int32_t)std::max<int64_t>(256, (opt.panel_bytes > 0 ? opt.panel_bytes : (int64_t)(2 << 20)) / (kt * 4)) : 1);
 
     int kernel = want;
     if (kernel == SDDMM_KERNEL_AUTO) kernel = SDDMM_KERNEL_HYBRID;
@@ -900,6 +1021,31 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     I.tile_size_x = (int32_t)std::min<int64_t>(n_cols, INT32_MAX);
     I.tile_size_y = (int32_t)std::min<int64_t>(n_rows, INT32_MAX);
     I.n_col_tiles = 1; I.n_row_panels = 1; I.n_blocks = 1; I.lanes_per_nnz = 8;
+
+    // The dense core first (HYBRID only, ranks the dense kernel's chunks divide, and only next to
+    // the non-compact tile streams, which can address a remainder): blocks of 128 ranked rows x
+    // 128 ranked columns filled to the threshold go to the matrix cores.
+    DenseBlocks D;
+    // Measured on the recommender shape it pays from K = 512 on (the remainder's shorter runs cost the
+    // tile kernel what the matrix cores save below that), so that is where "choose" turns it on.
+    const bool want_dense = opt.dense_blocks > 0 || (opt.dense_blocks < 0 && K >= 512);
+    if (kernel == SDDMM_KERNEL_HYBRID && want_dense && K % 32 == 0 && kt / 4 > 16 &&
+        (int64_t)n_rows * (K / 4) <= (int64_t)UINT32_MAX && (int64_t)n_cols * (K / 4) <= (int64_t)UINT32_MAX) {
+        const double threshold = (double)(opt.dense_permille > 0 ? opt.dense_permille : 300) / 1000.0;
+        const int64_t min_dense = opt.dense_min_nnz >= 0 ? opt.dense_min_nnz : std::max<int64_t>(nnz / 50, 1 << 20);
+        if (int rc = find_dense_blocks(n_rows, n_cols, nnz, row_ptr_all, col_ind_all, kDenseTile, threshold, min_dense, D)) return rc;
+        if (D.n_dense > 0) {
+            if (int rc = add_dense(c, D, vals)) return rc;
+            row_ptr = D.rem_row_ptr.data(); col_ind = D.rem_col.data(); nnz_part = nnz - D.n_dense;
+            c.row_ptr = row_ptr; c.col_ind = col_ind; c.nnz = nnz_part; c.orig = D.rem_orig.data();
+        }
+    }
+
+    // non-empty rows, ascending
+    std::vector<int32_t> ne;
+    ne.reserve((size_t)I.rows_touched);
+    for (int64_t r = 0; r < n_rows; ++r)
+        if (row_ptr[r + 1] > row_ptr[r]) ne.push_back((int32_t)r);
 
     if (kernel == SDDMM_KERNEL_HYBRID) {
         // Rows are split by length into classes:
@@ -929,81 +1075,59 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
             span = acc / (double)cnt;
         }
         const double tiles = std::max(1.0, span / std::max(1, x));
-        const int g_long = pick_tile_variant(kt, 0).G;
-        const bool have_g4 = env_i64("SDDMM_MED_CLASS", 0) != 0 && pick_tile_variant(kt, 4).G != 0 && g_long != 4;
-        int64_t long_min = (int64_t)std::max(2.0 * g_long, 2.0 * g_long * tiles);
+        const int g_long = pick_tile_variant(kt, opt.tile_lanes).G ? pick_tile_variant(kt, opt.tile_lanes).G : pick_tile_variant(kt, 0).G;
+        // rows with at least short_max nonzeros (2 per column tile with groups of 8 lanes) go to the tile kernel
         int64_t short_max = (int64_t)std::max(4.0, (g_long == 8 ? 2.0 : 1.0 * g_long) * tiles);
-        long_min = env_i64("SDDMM_LONG_ROW_MIN", long_min);
-        short_max = env_i64("SDDMM_SHORT_ROW_MAX", short_max);
-        if (!have_g4) long_min = short_max;
-        if (short_max > long_min) short_max = long_min;
-        std::vector<int32_t> rl, rm, rs;
-        int64_t nl = 0, nm = 0, nsh = 0;
+        if (opt.short_row_max >= 0) short_max = opt.short_row_max;
+        std::vector<int32_t> rl, rs;
+        int64_t nl = 0, nsh = 0;
         for (int32_t r : ne) {
             const int64_t d = row_ptr[r + 1] - row_ptr[r];
-            if (d >= long_min) { rl.push_back(r); nl += d; }
-            else if (d >= short_max) { rm.push_back(r); nm += d; }
+            if (d >= short_max) { rl.push_back(r); nl += d; }
             else { rs.push_back(r); nsh += d; }
         }
         // staging every H tile must be paid for by the nonzeros that use it
         const int64_t n_tiles_all = (n_cols + x - 1) / x;
         const int64_t stage_rows = std::max<int64_t>(n_tiles_all, c.cus) * x;
-        if (nl + nm < env_i64("SDDMM_STAGE_FACTOR", 8) * stage_rows) {
-            rs.insert(rs.end(), rl.begin(), rl.end()); rs.insert(rs.end(), rm.begin(), rm.end());
-            nsh += nl + nm; nl = nm = 0; rl.clear(); rm.clear();
+        if (nl < (opt.stage_factor >= 0 ? opt.stage_factor : 8) * stage_rows) {
+            rs.insert(rs.end(), rl.begin(), rl.end());
+            nsh += nl; nl = 0; rl.clear();
             std::sort(rs.begin(), rs.end());
         }
         // a small problem is one launch: splitting it only adds launch latency
-        if ((nl || nm) && nnz < env_i64("SDDMM_SPLIT_MIN_NNZ", 4 * 1000 * 1000)) {
-            rl.insert(rl.end(), rm.begin(), rm.end()); rl.insert(rl.end(), rs.begin(), rs.end());
-            nl += nm + nsh; nm = nsh = 0; rm.clear(); rs.clear();
+        if (nl && nnz_part < (opt.split_min_nnz >= 0 ? opt.split_min_nnz : (int64_t)4 * 1000 * 1000)) {
+            rl.insert(rl.end(), rs.begin(), rs.end());
+            nl += nsh; nsh = 0; rs.clear();
             std::sort(rl.begin(), rl.end());
         }
-        // a class too small to fill the machine joins its neighbour
-        if (!rm.empty() && nm * 50 < nnz) {
-            auto &dst = rl.empty() ? rs : rl;
-            dst.insert(dst.end(), rm.begin(), rm.end());
-            (rl.empty() ? nsh : nl) += nm; nm = 0; rm.clear();
-            std::sort(dst.begin(), dst.end());
+        // a class too small to fill the machine joins the other
+        if (!rl.empty() && !rs.empty() && nl * 50 < nnz_part) {
+            rs.insert(rs.end(), rl.begin(), rl.end());
+            nsh += nl; nl = 0; rl.clear();
+            std::sort(rs.begin(), rs.end());
         }
-        if (!rl.empty() && nl * 50 < nnz) {
-            auto &dst = rm.empty() ? rs : rm;
-            dst.insert(dst.end(), rl.begin(), rl.end());
-            (rm.empty() ? nsh : nm) += nl; nl = 0; rl.clear();
-            std::sort(dst.begin(), dst.end());
-        }
-        sddmm_plan_info scratch{};
         if (!rl.empty())
-            if (int rc = add_tile(c, rl, x, y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I, false, tile_x > 0)) return rc;
-        if (!rm.empty()) {
-            // (medium rows may use a narrower K slice: wider column tiles, longer runs, more passes)
-            int km = (int)env_i64("SDDMM_MED_KSLICE", kt == 128 ? 64 : kt);
-            int gm = (int)env_i64("SDDMM_MED_G", 4);
-            if (km <= 0 || km > kt || K % km || !pick_tile_variant(km, gm).G) { km = kt; gm = 4; }
-            const int32_t xm = km == kt ? x : (int32_t)std::min<int64_t>(kLdsMaxBytes / (km * 4), std::max<int64_t>(n_cols, 1));
-            if (int rc = add_tile(c, rm, xm, y_panel, gm, km, rl.empty() ? &I : &scratch, false, tile_x > 0 && km == kt)) return rc;
-        }
+            if (int rc = add_tile(c, rl, x, y_panel, opt.tile_lanes, kt, &I, false, tile_x > 0)) return rc;
         if (!rs.empty()) {
             // short rows: the padded, pipelined kernel reading H from global memory when the
             // rows are short enough for padding to stay cheap; the plain row gather otherwise
-            const int gg = (int)env_i64("SDDMM_GATHER_G", 8);
-            const bool padded = env_i64("SDDMM_GATHER_PADDED", 1) != 0 && pick_tile_variant(kt, gg).G != 0 &&
-                                (!rl.empty() || !rm.empty());
+            const int gg = opt.gather_lanes > 0 ? opt.gather_lanes : 8;
+            const bool padded = opt.gather_padded != 0 && pick_tile_variant(kt, gg).G != 0 && (!rl.empty() || D.n_dense > 0);
             if (padded) { if (int rc = add_tile(c, rs, 0, 0, gg, kt, nullptr, true)) return rc; }
             else if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
         }
-        I.kernel = (P->launches.size() == 1) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
-        I.class_nnz[0] = nl; I.class_nnz[1] = nm; I.class_nnz[2] = nsh;
-        I.class_rows[0] = (int64_t)rl.size(); I.class_rows[1] = (int64_t)rm.size(); I.class_rows[2] = (int64_t)rs.size();
+        I.kernel = (P->launches.size() == 1 && !P->launches[0].dfn) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
+        I.class_nnz[0] = nl; I.class_nnz[1] = 0; I.class_nnz[2] = nsh;
+        I.class_rows[0] = (int64_t)rl.size(); I.class_rows[1] = 0; I.class_rows[2] = (int64_t)rs.size();
     } else if (kernel == SDDMM_KERNEL_PANEL) {
         if (int rc = add_panel(c, ne, ks, tile_x, tile_y, &I)) return rc;
         I.kernel = kernel; I.class_nnz[1] = nnz; I.class_rows[1] = (int64_t)ne.size();
     } else if (kernel == SDDMM_KERNEL_LDS_TILE) {
         int32_t y = tile_y > 0 ? tile_y : (int32_t)std::min<int64_t>(std::max<int64_t>(n_rows, 1), INT32_MAX);
-        if (kt && env_i64("SDDMM_UNPADDED_TILE", 0) == 0) {
+        if (kt && opt.unpadded_tile <= 0) {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_t) : fit_t;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
-            if (int rc = add_tile(c, ne, x, tile_y > 0 ? tile_y : y_panel, (int)env_i64("SDDMM_TILE_G", 0), kt, &I, false, tile_x > 0)) return rc;
+            if (int rc = add_tile(c, ne, x, tile_y > 0 ? tile_y : y_panel, opt.tile_lanes, kt, &I, false, tile_x > 0)) return rc;
         } else {
             int32_t x = tile_x > 0 ? std::min(tile_x, fit_x) : fit_x;
             x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(n_cols, 1));
@@ -1011,8 +1135,8 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         }
         I.kernel = kernel; I.class_nnz[0] = nnz; I.class_rows[0] = (int64_t)ne.size();
     } else {
-        const int gg = (int)env_i64("SDDMM_GATHER_G", 0);
-        if (env_i64("SDDMM_ROW_PADDED", 0) != 0 && kt && pick_tile_variant(kt, gg).G != 0) {
+        const int gg = opt.gather_lanes > 0 ? opt.gather_lanes : 0;
+        if (opt.row_padded > 0 && kt && pick_tile_variant(kt, gg).G != 0) {
             if (int rc = add_tile(c, ne, 0, 0, gg, kt, &I, true)) return rc;
         } else if (int rc = add_row_gather(c, ne, true)) return rc;
         I.kernel = SDDMM_KERNEL_ROW_GATHER; I.class_nnz[2] = nnz; I.class_rows[2] = (int64_t)ne.size();
@@ -1031,27 +1155,60 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
 
 extern "C" {
 
-int sddmm_plan_create(const sddmm_coo *S, int32_t K, int32_t tile_size_x, int32_t tile_size_y, uint32_t flags,
-                      sddmm_plan **out)
+void sddmm_plan_options_init(sddmm_plan_options *opt)
+{
+    if (opt) default_options(*opt);
+}
+
+int sddmm_plan_get_options(const sddmm_plan *plan, sddmm_plan_options *opt)
+{
+    if (!plan || !opt) return fail(SDDMM_ERR_ARG, "sddmm_plan_get_options: NULL argument");
+    *opt = plan->options;
+    return SDDMM_OK;
+}
+
+int sddmm_plan_create_opt(const sddmm_coo *S, int32_t K, const sddmm_plan_options *opt_in, sddmm_plan **out)
 {
     if (!S || !out) return fail(SDDMM_ERR_ARG, "sddmm_plan_create: NULL argument");
     *out = nullptr;
-    if (S->sorted < 0) const_cast<sddmm_coo *>(S)->sorted = check_sorted(*S) ? 1 : 0;
     if (S->sorted != 1) return fail(SDDMM_ERR_UNSORTED, "sddmm_plan_create: matrix is not (row, col)-sorted; call sddmm_coo_sort_rows");
+    sddmm_plan_options opt;
+    default_options(opt);
+    if (opt_in) opt = *opt_in;
     try {
         std::vector<int32_t> rp;
         build_row_ptr(*S, rp);
-        return make_plan(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), S->vals.data(), nullptr, nullptr, K,
-                         tile_size_x, tile_size_y, flags, out);
-    } catch (const std::bad_alloc &) {
-        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create: out of host memory");
+        return make_plan(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), S->vals.data(), nullptr, nullptr, K, opt, out);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create: %s", e.what());
     }
+}
+
+int sddmm_plan_create(const sddmm_coo *S, int32_t K, int32_t tile_size_x, int32_t tile_size_y, uint32_t flags,
+                      sddmm_plan **out)
+{
+    sddmm_plan_options opt;
+    default_options(opt);
+    opt.kernel = (int32_t)(flags & 0xffu); opt.tile_size_x = tile_size_x; opt.tile_size_y = tile_size_y;
+    return sddmm_plan_create_opt(S, K, &opt, out);
 }
 
 int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
                              const int32_t *d_col_ind, int32_t K, int32_t tile_size_x, int32_t tile_size_y,
                              uint32_t flags, sddmm_plan **out)
 {
+    sddmm_plan_options opt;
+    default_options(opt);
+    opt.kernel = (int32_t)(flags & 0xffu); opt.tile_size_x = tile_size_x; opt.tile_size_y = tile_size_y;
+    return sddmm_plan_create_device_opt(n_rows, n_cols, nnz, d_row_ptr, d_col_ind, K, &opt, out);
+}
+
+int sddmm_plan_create_device_opt(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                                 const int32_t *d_col_ind, int32_t K, const sddmm_plan_options *opt_in, sddmm_plan **out)
+{
+    sddmm_plan_options opt;
+    default_options(opt);
+    if (opt_in) opt = *opt_in;
     if (!out) return fail(SDDMM_ERR_ARG, "sddmm_plan_create_device: out is NULL");
     *out = nullptr;
     if (n_rows < 0 || n_cols < 0 || nnz < 0 || !d_row_ptr || (nnz > 0 && !d_col_ind))
@@ -1080,10 +1237,9 @@ int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const 
             if (c == 2) return fail(SDDMM_ERR_RANGE, "sddmm_plan_create_device: a column index lies outside the matrix");
             if (c == 3) return fail(SDDMM_ERR_UNSORTED, "sddmm_plan_create_device: columns are not sorted inside a row");
         }
-        return make_plan(n_rows, n_cols, nnz, rp.data(), ci.data(), nullptr, d_row_ptr, d_col_ind, K, tile_size_x, tile_size_y,
-                         flags, out);
-    } catch (const std::bad_alloc &) {
-        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create_device: out of host memory");
+        return make_plan(n_rows, n_cols, nnz, rp.data(), ci.data(), nullptr, d_row_ptr, d_col_ind, K, opt, out);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_create_device: %s", e.what());
     }
 }
 
@@ -1123,6 +1279,13 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
             pa.accumulate = k_off > 0;
             hipLaunchKernelGGL(L.pfn, dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, pa);
         }
+    } else if (L.dfn) {
+        DenseArgs da = L.da;
+        da.nz_val = d_val ? nullptr : L.sval;
+        da.val = val;
+        da.W = d_W; da.H = d_H; da.out = d_out;
+        da.residual = residual;
+        hipLaunchKernelGGL(L.dfn, dim3((unsigned)L.grid), dim3((unsigned)L.block), 0, stream, da);
     } else if (L.tfn) {
         TileArgs ta = L.ta;
         ta.val = val;
@@ -1223,7 +1386,7 @@ int sddmm_execute_profiled(const sddmm_plan *plan, const float *d_val, const flo
         float ms = 0.f;
         HIP_TRY(hipEventElapsedTime(&ms, ev[i], ev[i + 1]));
         prof[i].kernel = L.kind;
-        prof[i].lanes_per_nnz = L.kind == SDDMM_KERNEL_PANEL ? 8 : (L.tfn ? L.tile_g : L.gather_g);
+        prof[i].lanes_per_nnz = L.dfn ? 0 : L.kind == SDDMM_KERNEL_PANEL ? 8 : (L.tfn ? L.tile_g : L.gather_g);
         prof[i].k_slice = L.k_slice;
         prof[i].n_kernel_launches = (L.k_slice > 0 && L.k_slice < plan->info.K) ? plan->info.K / L.k_slice : 1;
         prof[i].nnz = L.nnz;

@@ -12,7 +12,7 @@ struct sddmm_coo {
     int64_t n_rows = 0, n_cols = 0, nnz = 0;
     std::vector<int32_t> rows, cols;
     std::vector<float> vals;
-    int sorted = -1;  // -1 unknown, 0 no, 1 (row, col)-sorted
+    int sorted = 0;  // 1: (row, col)-sorted.  Set by whatever creates or reorders the matrix, never lazily.
 };
 
 // Tile-order view of a sorted matrix: tiles ascending, rows ascending inside a
@@ -43,6 +43,10 @@ int hw_threads();
 void parallel_ranges(int64_t n, int64_t grain,
                      const std::function<void(int64_t, int64_t, int)> &f, int *n_used = nullptr);
 
+// Runs f(begin, end, thread_index) over [0, n) in chunks of `chunk` that the threads
+// take in turn from a shared counter (for work of uneven cost per index).
+void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t, int64_t, int)> &f);
+
 bool check_sorted(const sddmm_coo &S);
 // CSR row pointers of a sorted matrix (n_rows+1 entries).
 void build_row_ptr(const sddmm_coo &S, std::vector<int32_t> &row_ptr);
@@ -51,5 +55,28 @@ void build_row_ptr(const sddmm_coo &S, std::vector<int32_t> &row_ptr);
 int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr,
                  const int32_t *col_ind, int32_t tile_x, int32_t tile_y, sddmm_tiling &T,
                  const int32_t *row_list, int64_t n_list);
+
+// The dense core of a sorted matrix, cut out for the dense-block kernel: blocks of `tile`
+// rows of similar length x `tile` columns that at least the threshold share of those rows
+// have, each listed with its nonzeros; everything else is left as a CSR remainder with a map
+// back to the positions in the original S.
+struct DenseBlocks {
+    int32_t tile = 0;
+    std::vector<int32_t> row_ids;   // [n_row_blocks * tile] rows in rank order (padded with row_ids[0])
+    std::vector<int32_t> col_ids;   // [n_tiles * tile] columns of each block, ascending (a short group repeats its last one)
+    std::vector<int32_t> tile_rb;   // [n_tiles] row block of each block; blocks of a row block are consecutive
+    std::vector<int32_t> tile_ptr;  // [n_tiles + 1]
+    std::vector<int32_t> nz_p;      // [n_dense] position in the original S
+    std::vector<uint16_t> nz_rc;    // [n_dense] (row in block << 8) | column in block
+    int64_t n_dense = 0;
+    // the remainder, rows as in S
+    std::vector<int32_t> rem_row_ptr;  // [n_rows + 1]
+    std::vector<int32_t> rem_col;      // [nnz - n_dense]
+    std::vector<int32_t> rem_orig;     // [nnz - n_dense] position in the original S
+};
+// threshold: least share of a block's rows that must have a column for it to be dense there.  Leaves D.n_dense == 0
+// (and the remainder arrays empty) when fewer than min_dense nonzeros would qualify.
+int find_dense_blocks(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr, const int32_t *col_ind,
+                      int32_t tile, double threshold, int64_t min_dense, DenseBlocks &D);
 
 }  // namespace sddmm

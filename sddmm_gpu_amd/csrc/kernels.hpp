@@ -2,6 +2,7 @@
 // and the kernel translation units.
 #pragma once
 #include <cstdint>
+#include <hip/hip_vector_types.h>
 
 namespace sddmm {
 
@@ -122,6 +123,27 @@ struct PanelVariant {
 using PanelFn = void (*)(const PanelArgs);
 PanelVariant pick_panel_variant(int k_slice);
 PanelFn panel_kernel(const PanelVariant &v);
+
+// Dense-block kernel: blocks of kDenseTile listed rows x kDenseTile listed columns computed
+// whole on the matrix cores; the block's nonzeros pick their results.
+constexpr int kDenseTile = 128;
+struct DenseArgs {
+    // Workgroup b takes slots b, b + grid, ...; a workgroup's filled slots come first.
+    const int32_t *slot_rows;  // [n_slots][kDenseTile] rows of the slot's block (a short row block padded with a valid row)
+    const int32_t *slot_cols;  // [n_slots][kDenseTile] its columns
+    const int2 *slot_range;    // [n_slots] the block's nonzeros in nz_*: [x, y); x == y: empty slot
+    const int32_t *nz_p;      // sorted position of each nonzero
+    const uint16_t *nz_rc;    // (row inside the block << 8) | column inside the block
+    const float *nz_val;      // values in list order or null
+    const float *val;         // values in sorted order or null (both null: no scaling)
+    const float *W, *H;
+    float *out;
+    int32_t n_slots;
+    int32_t K;                // row length of W and H, a multiple of 32
+    int32_t residual;         // 0: out = val * dot;  1: out = val - dot
+};
+using DenseFn = void (*)(const DenseArgs);
+DenseFn dense_kernel();
 
 // lanes per nonzero and float4 slots per lane for a given K (K % 4 == 0); G == 0: none
 Variant pick_variant(int K, bool lds_tile);

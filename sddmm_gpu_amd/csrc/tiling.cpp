@@ -153,7 +153,6 @@ extern "C" int sddmm_tiling_create(const sddmm_coo *S, int32_t tile_size_x, int3
 {
     if (!S || !out) return fail(SDDMM_ERR_ARG, "sddmm_tiling_create: NULL argument");
     *out = nullptr;
-    if (S->sorted < 0) const_cast<sddmm_coo *>(S)->sorted = check_sorted(*S) ? 1 : 0;
     if (S->sorted != 1) return fail(SDDMM_ERR_UNSORTED, "sddmm_tiling_create: matrix is not (row, col)-sorted");
     sddmm_tiling *T = new (std::nothrow) sddmm_tiling;
     if (!T) return fail(SDDMM_ERR_NOMEM, "sddmm_tiling_create: out of memory");

@@ -1,7 +1,9 @@
 """The sddmm command-line driver on the GPU: the reference's calling
 convention (sddmm input K tile_size_X tile_size_Y), its three output lines,
-and the result checked through the --json checksum against the CPU oracle run
-with the reference's own dense factors (0.1*drand48())."""
+and the result checked per nonzero (--check-against) with the vector the CPU
+oracle computes from the reference's own dense factors (0.1*drand48()), as the
+reference's optional check does (sddmm.cu:133-141); --check repeats it against
+the library's own CPU path."""
 import json
 import os
 import re
@@ -26,12 +28,24 @@ def test_cli_matches_oracle(oracle, tmp_path):
     S.write_mtx(mtx)
     K = 64
     W = oracle.initial(d["n_rows"], K); H = oracle.initial(d["n_cols"], K)
-    expect = oracle.sddmm_csr(d["row_ptr"].numpy(), cols, vals, W, H).astype(np.float64).sum()
-    for extra, tx, ty in (([], 192, 50000), (["--kernel", "row"], 0, 0), (["--kernel", "lds"], 64, 32)):
-        r = subprocess.run([CLI, str(mtx), str(K), str(tx), str(ty), "--json", "--runs", "3"] + extra, capture_output=True,
-                           text=True, timeout=120)
-        assert r.returncode == 0, r.stderr
+    cpu = oracle.sddmm_csr(d["row_ptr"].numpy(), cols, vals, W, H)
+    expect = cpu.astype(np.float64).sum()
+    vec = tmp_path / "oracle.f32"
+    cpu.tofile(vec)
+    for extra, tx, ty in (([], 192, 50000), (["--kernel", "row"], 0, 0), (["--kernel", "lds"], 64, 32),
+                          (["--kernel", "panel", "--ref-order"], 32, 64), (["--kernel", "hybrid", "--check"], 0, 0)):
+        dump = tmp_path / "out.f32"
+        r = subprocess.run([CLI, str(mtx), str(K), str(tx), str(ty), "--json", "--runs", "3", "--check-against", str(vec),
+                            "--dump-out", str(dump)] + extra, capture_output=True, text=True, timeout=120)
+        assert r.returncode == 0, r.stderr + r.stdout
         out = r.stdout
+        assert re.search(r"diff values in CPU and GPU: 0 ", out), out
+        got = np.fromfile(dump, np.float32)
+        assert got.shape == cpu.shape and np.all(np.abs(got - cpu) <= 1e-5 * np.sqrt(K) * np.abs(cpu) + 1e-6)
+        if "--ref-order" in extra:
+            assert re.search(r"Tilesize: X = 64, tilesize: Y = \d+", out), out
+        if "--check" in extra:
+            assert "Time for CPU SDDMM with K = 64" in out
         m = re.search(r"Matrix info:\s+rows: (\d+), cols: (\d+), nnz: (\d+)", out)
         assert m and tuple(map(int, m.groups())) == (d["n_rows"], d["n_cols"], d["nnz"])
         assert re.search(r"Tilesize: X = \d+, tilesize: Y = \d+, TB: \d+", out)
@@ -39,7 +53,13 @@ def test_cli_matches_oracle(oracle, tmp_path):
         assert m and int(m.group(1)) == K and float(m.group(2)) > 0
         js = json.loads([ln for ln in out.splitlines() if ln.startswith("{")][0])
         assert js["nnz"] == d["nnz"] and js["K"] == K
+        assert js["mismatches"] == 0 and js["max_rel"] <= 1e-5 * np.sqrt(K)
         assert abs(js["checksum"] - expect) <= 1e-5 * np.sqrt(K) * abs(expect) + 1e-6, (js["checksum"], expect)
+    # a permuted or perturbed result must be caught per nonzero although its checksum is the same
+    bad = cpu.copy(); bad[[3, 7]] = bad[[7, 3]]
+    bad.tofile(vec)
+    r = subprocess.run([CLI, str(mtx), str(K), "0", "0", "--check-against", str(vec)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and re.search(r"diff values in CPU and GPU: [12] ", r.stdout), r.stdout
 
 
 def test_cli_column_sorted_input_and_errors(oracle, tmp_path):
@@ -51,14 +71,17 @@ def test_cli_column_sorted_input_and_errors(oracle, tmp_path):
     vals = rng.random(len(keys)).astype(np.float32) + 0.5
     p = tmp_path / "colsorted.mtx"
     capi.Coo.from_arrays(n, m, rows[order], cols[order], vals[order]).write_mtx(p)
-    r = subprocess.run([CLI, str(p), "32", "16", "8", "--transpose", "--json"], capture_output=True, text=True, timeout=120)
-    assert r.returncode == 0, r.stderr
-    assert f"rows: {m}, cols: {n}, nnz: {len(keys)}" in r.stdout
     t_r, t_c, t_v, rp = oracle.transpose_sort(rows[order], cols[order], vals[order], m)
     W = oracle.initial(m, 32); H = oracle.initial(n, 32)
-    expect = oracle.sddmm_csr(rp, t_c, t_v, W, H).astype(np.float64).sum()
+    cpu = oracle.sddmm_csr(rp, t_c, t_v, W, H)
+    vec = tmp_path / "oracle_t.f32"
+    cpu.tofile(vec)
+    r = subprocess.run([CLI, str(p), "32", "16", "8", "--transpose", "--json", "--check-against", str(vec)], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 0, r.stderr + r.stdout
+    assert f"rows: {m}, cols: {n}, nnz: {len(keys)}" in r.stdout
     js = json.loads([ln for ln in r.stdout.splitlines() if ln.startswith("{")][0])
-    assert abs(js["checksum"] - expect) <= 1e-4 * abs(expect)
+    assert js["mismatches"] == 0
     # errors: missing file, bad K
     r = subprocess.run([CLI, str(tmp_path / "nope.mtx"), "32", "0", "0"], capture_output=True, text=True, timeout=60)
     assert r.returncode != 0 and "cannot open" in r.stderr

@@ -42,7 +42,7 @@ def test_full_size(oracle, cfg, K):
     del key
 
     out, info = run(d, capi.KERNEL_AUTO)
-    assert info["nnz"] == nnz and sum(info["class_nnz"]) == nnz
+    assert info["nnz"] == nnz and info["dense_nnz"] + sum(info["class_nnz"]) == nnz
     assert bool(torch.isfinite(out).all())
 
     # (1) a random sample of nonzeros against the CPU oracle

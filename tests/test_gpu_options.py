@@ -1,0 +1,122 @@
+"""Plans built from the options structure (sddmm_plan_create_opt): the same plan as
+the environment override layer gives, the unpadded and sub-list launches after
+sddmm_plan_set_values, and the dense-block launch on the matrix cores in every value
+mode and epilogue."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import parity_report
+from sddmm_gpu_amd import capi, synth
+from test_gpu_parity import check, residual_ok
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def host_plan(d, K, **opt):
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    return S.plan(K, options=capi.PlanOptions.defaults(ignore_env=1, **opt))
+
+
+def test_options_equal_environment_overrides(monkeypatch):
+    d = synth.make(3, 0.05, K=128, seed=5)
+    a = host_plan(d, 128, split_min_nnz=0, short_row_max=40, tile_short_batches=0)
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+    monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", "40")
+    monkeypatch.setenv("SDDMM_TILE_SHORT", "0")
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    b = S.plan(128)
+    ia, ib = a.info(), b.info()
+    for k in ia:
+        if k != "plan_ms":
+            assert ia[k] == ib[k], k
+    ob = b.options()
+    assert ob["split_min_nnz"] == 0 and ob["short_row_max"] == 40 and ob["tile_short_batches"] == 0  # reported back
+    # ignore_env: the same call with the variables still set builds the default plan
+    c = S.plan(128, options=capi.PlanOptions.defaults(ignore_env=1))
+    assert c.options()["short_row_max"] == -1
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev)
+    oa = torch.empty(d["nnz"], device=dev); ob_ = torch.empty(d["nnz"], device=dev)
+    a.execute(0, W.data_ptr(), H.data_ptr(), oa.data_ptr())
+    b.execute(0, W.data_ptr(), H.data_ptr(), ob_.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(oa, ob_)
+
+
+@pytest.mark.parametrize("K", [96, 100])
+def test_set_values_reaches_the_unpadded_lds_tile_launch(oracle, K):
+    # a K without a padded tile variant: the LDS_TILE plan is the unpadded stream kernel, which
+    # keeps its own stream-order copy of the values
+    d = synth.uniform_random(700, 900, 0.03, K=K, seed=70 + K)
+    plan = host_plan(d, K, kernel=capi.KERNEL_LDS_TILE, tile_size_x=64, unpadded_tile=1)
+    assert plan.info()["kernel"] == capi.KERNEL_LDS_TILE
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev); out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    check(d, out.cpu().numpy(), oracle, K)
+    dv2 = (d["val"] * 2.0 + 1.0).to(dev)
+    plan.set_values(dv2.data_ptr())
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    d2 = dict(d); d2["val"] = d["val"] * 2.0 + 1.0
+    check(d2, out.cpu().numpy(), oracle, K)
+
+
+def test_set_values_reaches_the_row_gather_sublist_launch(oracle):
+    # hybrid plan whose short class is the plain row gather over a list of rows (its own permuted stream)
+    K = 64
+    d = synth.make(3, 0.02, K=K, seed=8)
+    plan = host_plan(d, K, kernel=capi.KERNEL_HYBRID, split_min_nnz=0, short_row_max=30, gather_padded=0, stage_factor=0)
+    info = plan.info()
+    assert info["class_nnz"][0] > 0 and info["class_nnz"][2] > 0
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev); out = torch.full((d["nnz"],), float("nan"), device=dev)
+    dv2 = (d["val"] * 0.5 - 3.0).to(dev)
+    plan.set_values(dv2.data_ptr())
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    d2 = dict(d); d2["val"] = d["val"] * 0.5 - 3.0
+    check(d2, out.cpu().numpy(), oracle, K)
+
+
+@pytest.mark.parametrize("cfg,scale,K", [(3, 0.06, 128), (2, 1.0, 256), (3, 0.03, 512), (3, 0.03, 32)])
+def test_dense_block_launch(oracle, cfg, scale, K):
+    """The dense core on the matrix cores (fp32 MFMA), the remainder through the tile and gather
+    launches: no values, values at execute, values owned by the plan, and the residual epilogue."""
+    d = synth.make(cfg, scale, K=K)
+    dev = torch.device(DEV)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
+    opts = capi.PlanOptions.defaults(kernel=capi.KERNEL_HYBRID, dense_blocks=1, dense_min_nnz=1000, split_min_nnz=0, ignore_env=1)
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, keep=(rp, ci),
+                                     options=opts)
+    info = plan.info()
+    if K == 32:
+        assert info["dense_nnz"] == 0  # (the compact tile stream of narrow slices cannot address a remainder)
+    else:
+        assert info["dense_nnz"] > d["nnz"] // 10 and info["dense_blocks"] > 0, info
+    assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]
+    W = d["W"].to(dev); H = d["H"].to(dev); dv = d["val"].to(dev)
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    cpu1 = oracle.sddmm_coo(rows, cols, vals, d["W"].numpy(), d["H"].numpy(), apply_val=False)
+    _, absp1 = oracle.sddmm_f64(rows, cols, np.ones_like(vals), d["W"].numpy(), d["H"].numpy())
+    assert parity_report(out.cpu().numpy(), cpu1, K, absp1)["violations"] == 0
+    out.fill_(float("nan"))
+    plan.execute(dv.data_ptr(), W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    check(d, out.cpu().numpy(), oracle, K)
+    plan.set_values(dv.data_ptr())
+    out2 = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    for src in (0, dv.data_ptr()):
+        out.fill_(float("nan"))
+        plan.execute_epilogue(src, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
+        torch.cuda.synchronize()
+        residual_ok(out.cpu().numpy(), d, oracle, K)

@@ -68,7 +68,7 @@ def test_config2_bag_of_words(oracle, kernel, tx, ty):
     if kernel == "lds":
         assert info["kernel"] == capi.KERNEL_LDS_TILE and info["tile_size_x"] == 64
     if kernel == "auto":
-        assert sum(info["class_nnz"]) == d["nnz"] and sum(info["class_rows"]) == info["rows_touched"]
+        assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"] and sum(info["class_rows"]) == info["rows_touched"]
     print(info, rep)
 
 
@@ -155,7 +155,7 @@ def test_extreme_shapes_through_the_planner(oracle, monkeypatch, forced):
         for kernel in ("auto", "hybrid"):
             out, info = run_gpu(d, kernel=KERNELS[kernel])
             rep = check(d, out, oracle)
-            assert sum(info["class_nnz"]) == d["nnz"], (name, kernel, info)
+            assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"], (name, kernel, info)
 
 
 def test_empty_matrix_and_empty_rows(oracle):
@@ -220,16 +220,12 @@ def test_value_sources_and_host_form(oracle):
         plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
         d2 = dict(d); d2["val"] = d["val"] * 2.0
         check(d2, out.cpu().numpy(), oracle)
-    # the same on a hybrid plan with all three row classes
-    import os
-    os.environ.update(SDDMM_LONG_ROW_MIN="150", SDDMM_SHORT_ROW_MAX="15", SDDMM_SPLIT_MIN_NNZ="0", SDDMM_MED_CLASS="1")
-    try:
-        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, 0, 0,
-                                         capi.KERNEL_HYBRID, keep=(rp, ci))
-    finally:
-        for k in ("SDDMM_LONG_ROW_MIN", "SDDMM_SHORT_ROW_MAX", "SDDMM_SPLIT_MIN_NNZ", "SDDMM_MED_CLASS"):
-            os.environ.pop(k)
-    assert sum(plan.info()["class_nnz"]) == d["nnz"]
+    # the same on a hybrid plan with both row classes, built from the options structure
+    opts = capi.PlanOptions.defaults(kernel=capi.KERNEL_HYBRID, short_row_max=15, split_min_nnz=0, stage_factor=0, ignore_env=1)
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), 64, keep=(rp, ci),
+                                     options=opts)
+    assert plan.info()["class_nnz"][0] > 0 and plan.info()["class_nnz"][2] > 0
+    i_ = plan.info(); assert i_["dense_nnz"] + sum(i_["class_nnz"]) == d["nnz"]
     plan.set_values(dv.data_ptr())
     plan.execute(0, Wd.data_ptr(), Hd.data_ptr(), out.data_ptr())
     check(d, out.cpu().numpy(), oracle)
@@ -357,24 +353,22 @@ def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
             assert parity_report(out, base, d["K"], absp)["violations"] == 0, (kernel, tx, ty)
 
 
-@pytest.mark.parametrize("long_min,short_max", [(200, 20), (100, 100), (10 ** 9, 30), (50, 0)])
-def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
-    """Forces the three row classes (long: tile kernel, medium: tile kernel with
-    groups of 4 lanes in two K slices of 64, short: padded gather) of a hybrid plan
-    through the length thresholds and checks the union of their outputs."""
-    monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(long_min))
+@pytest.mark.parametrize("short_max", [20, 100, 10 ** 9, 0])
+def test_hybrid_row_classes(oracle, monkeypatch, short_max):
+    """Forces the two row classes of a hybrid plan (long: tile kernel, short: padded
+    gather) through the length threshold and checks the union of their outputs."""
     monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
     monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # split even this small matrix
-    monkeypatch.setenv("SDDMM_MED_CLASS", "1")      # the medium class is off by default
+    monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")
     d = synth.make(3, 0.02, K=128)
     deg = np.diff(d["row_ptr"].numpy())
     out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID)
     check(d, out, oracle)
-    assert sum(info["class_nnz"]) == d["nnz"]
+    assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]
     assert sum(info["class_rows"]) == int((deg > 0).sum())
-    if long_min == 200 and short_max == 20:
-        assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 4  # 1 + 2 K slices + 1
-        assert info["class_rows"][0] == int((deg >= 200).sum())
+    if short_max == 20:
+        assert info["kernel"] == capi.KERNEL_HYBRID and info["n_launches"] == 2
+        assert info["class_rows"][0] == int((deg >= 20).sum())
 
 
 @pytest.mark.parametrize("K,env", [
@@ -382,9 +376,9 @@ def test_hybrid_row_classes(oracle, monkeypatch, long_min, short_max):
     (128, {"SDDMM_TILE_WAVES": "16"}),                      # 16 instead of 12 waves per workgroup
     (128, {"SDDMM_TILE_ASSIGN": "1"}), (128, {"SDDMM_TILE_ASSIGN": "0"}),   # other work assignments
     (256, {"SDDMM_TILE_KSLICE": "256"}),                    # one full-K slice: variant G=16, 4 float4 per lane
-    (512, {"SDDMM_TILE_KSLICE": "256"}),                    # two slices of 256
-    (512, {"SDDMM_TILE_KSLICE": "512"}),                    # variant G=16 or 32
-    (128, {"SDDMM_MED_CLASS": "1", "SDDMM_LONG_ROW_MIN": "400"}),   # third class: groups of 4 lanes, K slices of 64
+    (512, {"SDDMM_TILE_KSLICE": "256", "SDDMM_DENSE": "0"}),                    # two slices of 256
+    (512, {"SDDMM_TILE_KSLICE": "512", "SDDMM_DENSE": "0"}),                    # variant G=16 or 32
+    (128, {"SDDMM_TILE_G": "4"}),                           # groups of 4 lanes in the tile kernel
     (128, {"SDDMM_GATHER_G": "4"}), (256, {"SDDMM_GATHER_PADDED": "0"}),
 ])
 def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
@@ -396,8 +390,8 @@ def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
     d = synth.make(3, 0.06, K=K, seed=77)
     out, info = run_gpu(d, kernel=capi.KERNEL_AUTO)
     check(d, out, oracle)
-    assert sum(info["class_nnz"]) == d["nnz"]
-    assert info["kernel"] == capi.KERNEL_HYBRID and info["class_nnz"][0] > 0 and info["class_nnz"][2] > 0, info
+    assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]
+    assert info["kernel"] == capi.KERNEL_HYBRID and info["class_nnz"][0] + info["dense_nnz"] > 0 and info["class_nnz"][2] > 0, info
     # the same plan with the values handed over once must give the same bits
     dev = torch.device("cuda:0")
     dd = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
@@ -445,7 +439,7 @@ def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
     if seed % 2:
         monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
         monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")  # tile even where staging the H tiles does not pay
-        monkeypatch.setenv("SDDMM_LONG_ROW_MIN", str(int(rng.integers(2, 200))))
+        rng.integers(2, 200)  # (keeps the random stream of the cases that follow)
         monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(int(rng.integers(1, 40))))
     # rows of very unequal length: a few long ones, many short or empty ones
     deg = np.minimum(n_cols, (rng.pareto(1.2, n_rows) * rng.integers(1, 30)).astype(np.int64))
@@ -467,4 +461,4 @@ def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
     _, absp = oracle.sddmm_f64(rows_np, cols_np, vals, d["W"].numpy(), d["H"].numpy())
     rep = parity_report(out, cpu, K, absp)
     assert rep["violations"] == 0, (rep, n_rows, n_cols, K, kernel, tile_x, tile_y, info)
-    assert sum(info["class_nnz"]) == d["nnz"]
+    assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]

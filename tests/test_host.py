@@ -263,6 +263,88 @@ def test_tiling_matches_reference_header(oracle):
     assert t["max_active_rows"] == ref["max_active_rows"]
 
 
+@pytest.mark.parametrize("K,threads", [(1, 1), (7, 3), (32, 0), (100, 2)])
+def test_sddmm_cpu_is_the_oracle_bit_for_bit(oracle, K, threads):
+    # the library's own CPU path against the oracle's restatement of sddmm_CPU_CSR (sddmm.cu:153-177)
+    rng = np.random.default_rng(K)
+    n_rows, n_cols = 300, 211
+    rows, cols = rand_coo(rng, n_rows, n_cols, 9000)
+    vals = rng.uniform(-2, 2, len(rows)).astype(np.float32)
+    W = rng.uniform(-1, 1, (n_rows, K)).astype(np.float32)
+    H = rng.uniform(-1, 1, (n_cols, K)).astype(np.float32)
+    S = capi.Coo.from_arrays(n_rows, n_cols, rows, cols, vals)
+    got = S.cpu(K, W, H, threads)
+    rp = S.row_ptr()
+    want = oracle.sddmm_csr(rp, cols, vals, W, H)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_sddmm_cpu_config1_end_to_end(tmp_path, oracle):
+    # BASELINE config 1 (4096 x 4096, 1 % density, K = 32) through the file reader, the sort and the CPU path
+    from sddmm_gpu_amd import synth
+    d = synth.make(1)
+    S0 = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    path = tmp_path / "c1.mtx"
+    S0.write_mtx(path)
+    S = capi.Coo.read_mtx(path)
+    S.sort_rows()
+    r, c, v = S.arrays()
+    assert np.array_equal(r, d["row_ind"].numpy()) and np.array_equal(c, d["col_ind"].numpy())
+    W, H = d["W"].numpy(), d["H"].numpy()
+    got = S.cpu(32, W, H)
+    want = oracle.sddmm_csr(d["row_ptr"].numpy(), c, v, W, H)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    f64 = (W[r].astype(np.float64) * H[c].astype(np.float64)).sum(1) * v
+    assert np.abs(got - f64).max() <= 1e-5 * np.sqrt(32) * np.abs(f64).max()
+
+
+def test_cli_cpu_only_matches_oracle_per_nonzero(tmp_path, oracle):
+    # the command-line tool without a GPU: reader, sort, CPU path, per-nonzero check against the oracle's vector
+    import subprocess
+    cli = os.path.join(ROOT, "sddmm_gpu_amd", "bin", "sddmm")
+    rng = np.random.default_rng(11)
+    rows, cols = rand_coo(rng, 200, 150, 3000, sort=False)
+    vals = rng.uniform(0.5, 1.5, len(rows)).astype(np.float32)
+    S = capi.Coo.from_arrays(200, 150, rows, cols, vals)
+    mtx = tmp_path / "u.mtx"
+    S.write_mtx(mtx)
+    S.sort_rows()
+    r, c, v = S.arrays()
+    K = 32
+    want = oracle.sddmm_csr(S.row_ptr(), c, v, oracle.initial(200, K), oracle.initial(150, K))
+    vec = tmp_path / "want.f32"; want.tofile(vec)
+    dump = tmp_path / "got.f32"
+    p = subprocess.run([cli, str(mtx), str(K), "0", "0", "--cpu-only", "--cpu-threads", "2", "--check-against", str(vec),
+                        "--dump-out", str(dump), "--json"], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 0, p.stderr + p.stdout
+    assert "diff values in CPU and GPU: 0 " in p.stdout and "Time for CPU SDDMM with K = 32" in p.stdout
+    assert np.array_equal(np.fromfile(dump, np.float32).view(np.uint32), want.view(np.uint32))
+    (want * 1.001).astype(np.float32).tofile(vec)
+    p = subprocess.run([cli, str(mtx), str(K), "0", "0", "--cpu-only", "--check-against", str(vec)], capture_output=True, text=True,
+                       timeout=60)
+    assert p.returncode == 1
+
+
+def test_sddmm_cpu_errors():
+    S = capi.Coo.from_arrays(3, 3, [2, 0], [0, 1])  # unsorted
+    with pytest.raises(capi.SddmmError) as e:
+        S.cpu(4, np.zeros((3, 4), np.float32), np.zeros((3, 4), np.float32))
+    assert e.value.code == capi.ERR_UNSORTED
+    S.sort_rows()
+    assert capi.lib().sddmm_cpu(S.h, 0, None, None, None, 1) == capi.ERR_ARG
+    E = capi.Coo.from_arrays(3, 3, [], [])
+    assert len(E.cpu(4, np.zeros((3, 4), np.float32), np.zeros((3, 4), np.float32))) == 0
+
+
+def test_plan_options_defaults_mean_choose():
+    o = capi.PlanOptions.defaults()
+    d = o.as_dict()
+    assert d["kernel"] == capi.KERNEL_AUTO and d["tile_size_x"] == 0 and d["tile_size_y"] == 0 and d["ignore_env"] == 0
+    assert all(v == -1 for k, v in d.items() if k not in ("kernel", "tile_size_x", "tile_size_y", "ignore_env")), d
+    with pytest.raises(KeyError):
+        capi.PlanOptions.defaults(no_such_field=1)
+
+
 def test_plan_without_gpu_fails_loudly():
     n, arch = capi.device_info()
     if n > 0:
