@@ -8,7 +8,16 @@ Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps 1000] [--warmup 100] [--config 3] [--K 128]
                   [--kernel auto|row|lds|panel|hybrid] [--tile-x X] [--tile-y Y] [--spinup-ms 300]
-                  [--no-sweep] [--no-cpu] [--copy-probe]
+                  [--opt field=value ...] [--no-sweep] [--no-cpu] [--no-parity] [--copy-probe]
+                  [--tile-sweep] [--from-prof DIR]
+
+--tile-sweep adds one row per tile configuration (tile_size_x x K slice x lanes per nonzero,
+explicit values honoured) with its time, GB/s and launch shape; run under
+rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE the same rows get their LDS
+conflict counters (sddmm_gpu_amd/rocprof.py matches them by kernel variant, LDS size and grid).
+--from-prof DIR merges such a profile (HBM bytes per step scaled by the copy probe, LDS bank
+conflicts per active cycle, per-kernel durations) into the line; without it roofline.traffic is
+read from the summary of the same workload kept under profiles/, whose name the line gives.
 """
 import argparse
 import json
@@ -21,10 +30,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
-# the default workload (see profiles/*hbm_traffic*.txt for the runs and the
-# copy-kernel scale factors); None where no such measurement exists.
-MEASURED_TRAFFIC = {(3, 1.0, 128, "auto", 0, 0): 3.14e9}
+
+
+def traffic_profile_path(config, scale, K, kernel, tile_x, tile_y, opts):
+    """Where the rocprofv3 summary with this workload's HBM bytes per step is kept (made by
+    python -m sddmm_gpu_amd.rocprof from FETCH_SIZE / WRITE_SIZE passes of this script)."""
+    if scale != 1.0 or tile_x or tile_y or opts:
+        return None
+    return os.path.join(ROOT, "profiles", f"hbm_traffic_config{config}_k{K}_{kernel}.txt")
 
 
 def alg_bytes(nnz, n_rows, K, rows_touched, cols_touched):
@@ -67,23 +80,64 @@ def cpu_baseline(d, K, budget_s=12.0):
     H = d["H"].cpu().numpy()
     nnz = d["nnz"]
 
-    def run(n):
+    def run(n, reps):
         r = d["row_ind"][:n].cpu().numpy(); c = d["col_ind"][:n].cpu().numpy(); v = d["val"][:n].cpu().numpy()
+        oracle.sddmm_coo(r, c, v, W, H, nthreads=threads, apply_val=True, timed=True)  # warm-up, not timed
         best = None
-        for _ in range(2):
+        for _ in range(reps):
             _, sec = oracle.sddmm_coo(r, c, v, W, H, nthreads=threads, apply_val=True, timed=True)
             best = sec if best is None else min(best, sec)
         return best
 
     n0 = min(nnz, 1_000_000)
-    t = run(n0)
+    t = run(n0, 1)
     rate = n0 / max(t, 1e-9)
-    n = int(min(nnz, max(n0, rate * budget_s / 2)))
-    if n > n0:
-        t = run(n)
+    n = int(min(nnz, max(n0, rate * budget_s / 4)))  # one warm-up + three timed runs inside the budget
+    t = run(n, 3)
     gflops = 2.0 * n * K / t / 1e9
+    model = "unknown CPU"
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name"):
+                model = ln.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     return dict(value=round(gflops, 3), unit="GFLOP/s", cores=threads, kind="port",
-                sample=f"first {n} of {nnz} nonzeros (rows in order), K={K}, best of 2 runs, {t * 1e3:.1f} ms")
+                sample=f"first {n} of {nnz} nonzeros (rows in order), K={K}, one warm-up then best of 3 runs, "
+                       f"{t * 1e3:.1f} ms, {threads} threads on {model}")
+
+
+def parity_block(d, K, out, torch, n_sample=200_000):
+    """A seeded sample of the nonzeros against the CPU oracle, outside the timed region: the
+    strict count (|gpu - cpu| > 1e-5*sqrt(K)*|cpu|), the worst relative and norm-wise errors,
+    the count under the bound the parity tests assert (relative, or norm-wise for nonzeros
+    whose terms cancel), and how many of the oracle's own results miss the strict bound against
+    an fp64 sum (what fp32 summation order alone costs on this input)."""
+    import numpy as np
+    from oracle import oracle
+    g = torch.Generator(device=out.device); g.manual_seed(4242)
+    n = min(n_sample, d["nnz"])
+    idx = torch.randint(0, d["nnz"], (n,), generator=g, device=out.device)
+    rows = d["row_ind"][idx].cpu().numpy(); cols = d["col_ind"][idx].cpu().numpy(); vals = d["val"][idx].cpu().numpy()
+    # only the sampled rows of W and H travel to the host
+    ur, ri = np.unique(rows, return_inverse=True); uc, ci = np.unique(cols, return_inverse=True)
+    W = d["W"][torch.from_numpy(ur).to(out.device).long()].cpu().numpy()
+    H = d["H"][torch.from_numpy(uc).to(out.device).long()].cpu().numpy()
+    ri = ri.astype(np.int32); ci = ci.astype(np.int32)
+    cpu = oracle.sddmm_coo(ri, ci, vals, W, H).astype(np.float64)
+    f64, absp = oracle.sddmm_f64(ri, ci, vals, W, H)
+    gpu = out[idx].cpu().numpy().astype(np.float64)
+    tol = 1e-5 * np.sqrt(K)
+    diff = np.abs(gpu - cpu)
+    nz = np.abs(cpu) > 0; pos = absp > 0
+    return dict(n_sample=int(n), tol=tol,
+                strict_violations=int((diff > tol * np.abs(cpu)).sum()),
+                max_rel=float((diff[nz] / np.abs(cpu[nz])).max()) if nz.any() else 0.0,
+                max_normwise=float((diff[pos] / absp[pos]).max()) if pos.any() else 0.0,
+                violations=int((diff > tol * np.maximum(np.abs(cpu), absp / 100.0)).sum()),
+                cpu_vs_f64_strict=int((np.abs(cpu - f64) > tol * np.abs(f64)).sum()),
+                gpu_vs_f64_strict=int((np.abs(gpu - f64) > tol * np.abs(f64)).sum()))
 
 
 KERNEL_NAMES = {1: "row_gather", 2: "lds_tile", 3: "panel", 4: "hybrid", 5: "dense_block"}
@@ -108,6 +162,11 @@ def main():
     ap.add_argument("--tile-y", type=int, default=0)
     ap.add_argument("--no-sweep", action="store_true", help="skip the K = 32, 128, 256, 512 report")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-parity", action="store_true", help="skip the sampled comparison with the CPU oracle")
+    ap.add_argument("--opt", action="append", default=[], metavar="FIELD=VALUE",
+                    help="a field of sddmm_plan_options (include/sddmm.h), e.g. --opt k_slice=64 --opt dense_blocks=1")
+    ap.add_argument("--tile-sweep", action="store_true", help="one row per tile configuration (see the module docstring)")
+    ap.add_argument("--from-prof", default=None, metavar="DIR", help="merge a rocprofv3 profile of this workload into the line")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy (a known-size reference for HBM counters)")
     args = ap.parse_args()
@@ -127,6 +186,12 @@ def main():
     names = {1: "uniform 4096^2 1%", 2: "bag-of-words 1500x12419", 3: "recommender 480189x17770 ~100M nnz",
              4: "R-MAT 2^22 ~200M nnz", 5: "banded 2^20 64/row"}
 
+    opt_fields = {}
+    for kv in args.opt:
+        k, _, v = kv.partition("=")
+        opt_fields[k] = int(v)
+    executes = [0]
+
     d = synth.make(args.config, args.scale, device=dev, K=args.K)
     K0 = d["K"]
     sigma = float(d["W"].std())
@@ -138,10 +203,15 @@ def main():
             d["H"] = torch.randn(d["n_cols"], K, generator=g, device=dev) * sigma
             d["K"] = K
 
-    def measure(K):
+    def measure(K, steps=None, warmup=None, spinup=None, keep_out=False, **more):
         set_rank(K)
+        steps = args.steps if steps is None else steps
+        warmup = args.warmup if warmup is None else warmup
+        spinup = args.spinup_ms if spinup is None else spinup
+        fields = dict(kernel=kernel, tile_size_x=args.tile_x, tile_size_y=args.tile_y)
+        fields.update(opt_fields); fields.update(more)
         plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(),
-                                         d["col_ind"].data_ptr(), K, args.tile_x, args.tile_y, kernel)
+                                         d["col_ind"].data_ptr(), K, options=capi.PlanOptions.defaults(**fields))
         info = plan.info()
         out = torch.empty(d["nnz"], device=dev)
         # S.val belongs to the matrix like its indices: it is handed to the plan once,
@@ -150,21 +220,41 @@ def main():
         torch.cuda.synchronize()
         vp, wp, hp, op = 0, d["W"].data_ptr(), d["H"].data_ptr(), out.data_ptr()
         epi = capi.EPILOGUE_RESIDUAL if args.epilogue == "residual" else capi.EPILOGUE_SCALE
-        run = (lambda s: plan.execute(vp, wp, hp, op, s)) if args.epilogue == "scale" else \
-              (lambda s: plan.execute_epilogue(vp, wp, hp, op, epi, s))
-        wall, mean_ev, med_ev = time_steps(run, args.steps, args.warmup, torch,
-                                           args.spinup_ms)
+
+        def run(s):
+            executes[0] += 1
+            if args.epilogue == "scale":
+                plan.execute(vp, wp, hp, op, s)
+            else:
+                plan.execute_epilogue(vp, wp, hp, op, epi, s)
+
+        wall, mean_ev, med_ev = time_steps(run, steps, warmup, torch, spinup)
         prof = plan.execute_profiled(vp, wp, hp, op, torch.cuda.current_stream().cuda_stream)
+        executes[0] += 1
         flops = 2.0 * d["nnz"] * K
         balg = alg_bytes(d["nnz"], d["n_rows"], K, info["rows_touched"], info["cols_touched"])
         res = dict(K=K, ms_per_step=wall, kernel_ms_mean=mean_ev, kernel_ms_median=med_ev,
                    gflops=flops / (wall * 1e6), alg_bytes=balg, alg_gbps=balg / (mean_ev * 1e6),
-                   frac=balg / (mean_ev * 1e6) / HBM_PEAK_GBPS, info=info, prof=prof)
+                   frac=balg / (mean_ev * 1e6) / HBM_PEAK_GBPS, info=info, prof=prof, options=plan.options())
+        if keep_out:
+            if args.epilogue != "scale":
+                plan.execute(vp, wp, hp, op, torch.cuda.current_stream().cuda_stream)
+                executes[0] += 1
+            torch.cuda.synchronize()
+            res["out"] = out
         plan.close()
         return res
 
-    main_res = measure(K0)
+    main_res = measure(K0, keep_out=not args.no_parity)
     info = main_res["info"]
+    parity = None
+    if not args.no_parity:
+        parity = parity_block(d, K0, main_res.pop("out"), torch)
+    tpath = traffic_profile_path(args.config, args.scale, K0, args.kernel, args.tile_x, args.tile_y, opt_fields)
+    traffic = None
+    if tpath:
+        from sddmm_gpu_amd import rocprof
+        traffic = rocprof.traffic_from_profile_text(tpath)
     line = {
         "metric": "SDDMM GFLOP/s (2*nnz*K), fp32",
         "value": round(main_res["gflops"], 2),
@@ -183,16 +273,46 @@ def main():
                    "kernel": KERNEL_NAMES[info["kernel"]], "tile_size_x": info["tile_size_x"],
                    "tile_size_y": info["tile_size_y"], "k_slice": info["k_slice"],
                    "kernel_launches_per_step": info["n_launches"], "plan_ms": round(info["plan_ms"], 1),
-                   "spinup_ms": args.spinup_ms, "epilogue": args.epilogue},
+                   "spinup_ms": args.spinup_ms, "epilogue": args.epilogue,
+                   "dense_nnz": info["dense_nnz"], "dense_blocks": info["dense_blocks"],
+                   "plan_options": {k: v for k, v in main_res["options"].items() if v not in (-1, 0) or k == "kernel"}},
         "roofline": {"bound": "hbm", "achieved": round(main_res["alg_gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(main_res["frac"], 4),
-                     "traffic": MEASURED_TRAFFIC.get((args.config, args.scale, K0, args.kernel, args.tile_x, args.tile_y)),
+                     "traffic": traffic,
+                     "traffic_source": (os.path.relpath(tpath, ROOT) if traffic is not None else None),
                      "alg_bytes_per_step": main_res["alg_bytes"], "kernel_ms": round(main_res["kernel_ms_mean"], 5),
                      "kernels": [{"kernel": KERNEL_NAMES[p["kernel"]], "lanes_per_nnz": p["lanes_per_nnz"],
                                   "k_slice": p["k_slice"], "launches": p["n_kernel_launches"], "nnz": p["nnz"],
                                   "rows": p["rows"], "stream_positions": p["stream_positions"],
                                   "ms": round(p["ms"], 5)} for p in main_res["prof"]]},
     }
+    if parity is not None:
+        line["parity"] = parity
+    if args.tile_sweep:
+        # tile width x K slice x lanes per nonzero, explicit values honoured by the planner; fewer steps per row
+        rows = []
+        fit = {32: 1280, 64: 640, 128: 320}
+        for ks in (32, 64, 128):
+            if K0 % ks:
+                continue
+            for tx in sorted({fit[ks], fit[ks] // 2, 192}):
+                if tx > fit[ks]:
+                    continue
+                for g in (4, 8):
+                    try:
+                        r = measure(K0, steps=max(10, args.steps // 10), warmup=max(3, args.warmup // 10), spinup=30.0,
+                                    kernel=capi.KERNEL_LDS_TILE, tile_size_x=tx, k_slice=ks, tile_lanes=g)
+                    except capi.SddmmError as e:
+                        rows.append(dict(tile_size_x=tx, k_slice=ks, lanes_per_nnz=g, error=str(e)))
+                        continue
+                    i2 = r["info"]
+                    rows.append(dict(tile_size_x=i2["tile_size_x"], tile_size_y=i2["tile_size_y"], k_slice=i2["k_slice"],
+                                     lanes_per_nnz=i2["lanes_per_nnz"], n_col_tiles=i2["n_col_tiles"], lds_bytes=i2["lds_bytes"],
+                                     grid=i2["grid"], block=i2["block"], padded_positions=i2["padded_positions"],
+                                     ms=round(r["kernel_ms_mean"], 4), gflops=round(r["gflops"], 1),
+                                     alg_gbps=round(r["alg_gbps"], 1), hbm_frac=round(r["frac"], 4)))
+                    print("tile-sweep", rows[-1], file=sys.stderr, flush=True)
+        line["tile_sweep"] = rows
     if not args.no_sweep and args.config == 3:
         sweep = {}
         for K in (32, 128, 256, 512):
@@ -200,17 +320,19 @@ def main():
             sweep[str(K)] = {"gflops": round(r["gflops"], 1), "kernel_ms": round(r["kernel_ms_mean"], 4),
                              "hbm_frac": round(r["frac"], 4)}
         line["gflops_by_K"] = sweep
-    # a plain 1 GiB device-to-device copy next to it: with --copy-probe as the known-size
-    # reference for the HBM counters, always as the bandwidth a streaming kernel reaches here
+    # a plain 1 GiB copy kernel next to it (sddmm_copy_probe): with --copy-probe the known-size
+    # reference the HBM counters of a profile are scaled by, always the bandwidth a streaming
+    # kernel reaches on this device
     n = 1 << 30
     a = torch.empty(n // 4, device=dev); b = torch.empty_like(a)
     a.fill_(1.0)
-    b.copy_(a)
+    cs = torch.cuda.current_stream().cuda_stream
+    capi.copy_probe(a.data_ptr(), b.data_ptr(), n, cs)
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(10):
-        b.copy_(a)
+        capi.copy_probe(a.data_ptr(), b.data_ptr(), n, cs)
     e1.record()
     torch.cuda.synchronize()
     line["roofline"]["measured_copy_gbps"] = round(10 * 2.0 * n / (e0.elapsed_time(e1) * 1e6), 1)
@@ -220,6 +342,17 @@ def main():
     if not args.no_cpu:
         set_rank(K0)
         line["cpu_baseline"] = cpu_baseline(d, K0)
+    line["config"]["executes"] = executes[0]
+    line["config"]["argv"] = sys.argv[1:]
+    if args.from_prof:
+        from sddmm_gpu_amd import rocprof
+        s = rocprof.summarize(args.from_prof)
+        if s.get("traffic") is not None:
+            line["roofline"]["traffic"] = s["traffic"]
+            line["roofline"]["traffic_source"] = args.from_prof
+        line["roofline"]["lds_bank_conflict_per_active"] = s.get("lds_bank_conflict_per_active")
+        line["roofline"]["profile"] = {k: {f: e[f] for f in ("avg_us", "launches_per_step", "lds_bank_conflict_per_active",
+                                                             "fma_share_of_valu") if f in e} for k, e in s["kernels"].items()}
     print(json.dumps(line))
 
 
