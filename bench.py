@@ -165,6 +165,8 @@ def main():
     ap.add_argument("--no-parity", action="store_true", help="skip the sampled comparison with the CPU oracle")
     ap.add_argument("--opt", action="append", default=[], metavar="FIELD=VALUE",
                     help="a field of sddmm_plan_options (include/sddmm.h), e.g. --opt k_slice=64 --opt dense_blocks=1")
+    ap.add_argument("--plan-file", default=None, metavar="PATH",
+                    help="load the plan from PATH.k<K> when that file fits this matrix, K and options; otherwise build it and save it there")
     ap.add_argument("--tile-sweep", action="store_true", help="one row per tile configuration (see the module docstring)")
     ap.add_argument("--from-prof", default=None, metavar="DIR", help="merge a rocprofv3 profile of this workload into the line")
     ap.add_argument("--copy-probe", action="store_true",
@@ -210,14 +212,27 @@ def main():
         spinup = args.spinup_ms if spinup is None else spinup
         fields = dict(kernel=kernel, tile_size_x=args.tile_x, tile_size_y=args.tile_y)
         fields.update(opt_fields); fields.update(more)
-        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(),
-                                         d["col_ind"].data_ptr(), K, options=capi.PlanOptions.defaults(**fields))
+        popt = capi.PlanOptions.defaults(**fields)
+        plan, loaded = None, False
+        if args.plan_file and not more:
+            try:
+                plan = capi.Plan.load_device(f"{args.plan_file}.k{K}", d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(),
+                                             d["col_ind"].data_ptr(), K, options=popt)
+                loaded = True
+            except capi.SddmmError as e:
+                print(f"bench.py: no usable plan file ({e}); building the plan", file=sys.stderr)
+        if plan is None:
+            plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(),
+                                             d["col_ind"].data_ptr(), K, options=popt)
         info = plan.info()
+        info["plan_loaded"] = loaded
         out = torch.empty(d["nnz"], device=dev)
         # S.val belongs to the matrix like its indices: it is handed to the plan once,
         # outside the timed region; W and H are the per-step inputs
         plan.set_values(d["val"].data_ptr(), torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
+        if args.plan_file and not more and not loaded:
+            plan.save(f"{args.plan_file}.k{K}")
         vp, wp, hp, op = 0, d["W"].data_ptr(), d["H"].data_ptr(), out.data_ptr()
         epi = capi.EPILOGUE_RESIDUAL if args.epilogue == "residual" else capi.EPILOGUE_SCALE
 
@@ -272,7 +287,7 @@ def main():
                    "n_rows": d["n_rows"], "n_cols": d["n_cols"], "nnz": d["nnz"], "K": K0, "seed": d["seed"],
                    "kernel": KERNEL_NAMES[info["kernel"]], "tile_size_x": info["tile_size_x"],
                    "tile_size_y": info["tile_size_y"], "k_slice": info["k_slice"],
-                   "kernel_launches_per_step": info["n_launches"], "plan_ms": round(info["plan_ms"], 1),
+                   "kernel_launches_per_step": info["n_launches"], "plan_ms": round(info["plan_ms"], 1), "plan_loaded": info["plan_loaded"],
                    "spinup_ms": args.spinup_ms, "epilogue": args.epilogue,
                    "dense_nnz": info["dense_nnz"], "dense_blocks": info["dense_blocks"],
                    "plan_options": {k: v for k, v in main_res["options"].items() if v not in (-1, 0) or k == "kernel"}},

@@ -247,6 +247,27 @@ int sddmm_plan_create_device_opt(int64_t n_rows, int64_t n_cols, int64_t nnz, co
                                  sddmm_plan **out);
 int sddmm_plan_get_options(const sddmm_plan *plan, sddmm_plan_options *opt);
 
+/* Plan files: the tiling pass is the expensive part of setting up a large
+ * matrix (half a second at 10^8 nonzeros), so a plan can be written to a file
+ * next to the matrix's binary side-file and loaded back instead of being built
+ * again.  The file holds the plan's device arrays and launch descriptors under
+ * a key: matrix size, nnz, K, the plan options it was built with (tile sizes
+ * and kernel family among them) and a hash of the sparsity pattern.  Loading
+ * checks the key against the caller's matrix, K and options (opt == NULL: any
+ * options) and fails with SDDMM_ERR_FORMAT on a mismatch or on a file written
+ * by another build of the library.  sddmm_plan_load is the counterpart of
+ * sddmm_plan_create (the file carries the pattern and the values);
+ * sddmm_plan_load_device the one of sddmm_plan_create_device (the plan borrows
+ * the caller's device arrays again; the pattern hash is computed on the device).
+ * The reference's analogue are the ad-hoc dumps of its converted matrices,
+ * util.h:83-118.                                                             */
+int sddmm_plan_save(const sddmm_plan *plan, const char *path);
+int sddmm_plan_load(const char *path, const sddmm_coo *S, int32_t K, const sddmm_plan_options *opt,
+                    sddmm_plan **out);
+int sddmm_plan_load_device(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz,
+                           const int32_t *d_row_ptr, const int32_t *d_col_ind, int32_t K,
+                           const sddmm_plan_options *opt, sddmm_plan **out);
+
 /* Gives the plan its own copy of S.val (nnz fp32 in sorted order, device
  * pointer), laid out the way each of its kernels streams the nonzeros, so
  * that sddmm_execute(plan, NULL, ...) reads values coalesced.  This is what

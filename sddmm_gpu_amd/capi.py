@@ -102,6 +102,10 @@ SIGNATURES = {
     "sddmm_plan_create_device_opt": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int32, POINTER(PlanOptions),
                                              POINTER(c_void_p)]),
     "sddmm_plan_get_options": (c_int, [c_void_p, POINTER(PlanOptions)]),
+    "sddmm_plan_save": (c_int, [c_void_p, c_char_p]),
+    "sddmm_plan_load": (c_int, [c_char_p, c_void_p, c_int32, POINTER(PlanOptions), POINTER(c_void_p)]),
+    "sddmm_plan_load_device": (c_int, [c_char_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int32, POINTER(PlanOptions),
+                                       POINTER(c_void_p)]),
     "sddmm_plan_set_values": (c_int, [c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_get_info": (c_int, [c_void_p, POINTER(PlanInfo)]),
     "sddmm_plan_destroy": (None, [c_void_p]),
@@ -247,6 +251,12 @@ class Coo:
             check(lib().sddmm_plan_create(self.h, K, tile_x, tile_y, kernel, byref(h)))
         return Plan(h)
 
+    def load_plan(self, path, K, options=None):
+        """A plan saved by Plan.save for this matrix, K and options (None: any options)."""
+        h = c_void_p()
+        check(lib().sddmm_plan_load(str(path).encode(), self.h, K, byref(options) if options is not None else None, byref(h)))
+        return Plan(h)
+
     def cpu(self, K, W, H, n_threads=0):
         """The SDDMM on the host cores (sddmm_cpu): fp32, sequential sums, no GPU needed."""
         n_rows, n_cols, nnz, _ = self.info()
@@ -288,6 +298,16 @@ class Plan:
             check(lib().sddmm_plan_create_device(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K, tile_x,
                                                  tile_y, kernel, byref(h)))
         return cls(h, keep)
+
+    @classmethod
+    def load_device(cls, path, n_rows, n_cols, nnz, d_row_ptr, d_col_ind, K, options=None, keep=None):
+        h = c_void_p()
+        check(lib().sddmm_plan_load_device(str(path).encode(), n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), K,
+                                           byref(options) if options is not None else None, byref(h)))
+        return cls(h, keep)
+
+    def save(self, path):
+        check(lib().sddmm_plan_save(self.h, str(path).encode()))
 
     def options(self):
         o = PlanOptions()

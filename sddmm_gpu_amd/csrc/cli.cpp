@@ -35,7 +35,9 @@ static void usage()
             "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
             "  --kernel NAME  auto | row | lds | panel | hybrid\n"
             "  --runs N       timed repetitions (default 1; the median is printed)\n"
-            "  --save-bin F   write the parsed, sorted matrix to F for fast re-loading\n"
+            "  --save-bin F   write the parsed, sorted matrix to F for fast re-loading, and the plan built for\n"
+            "                 (K, tile sizes, kernel) beside it as F.k<K>.x<X>.y<Y>.<kernel>.plan; a later run on F with\n"
+            "                 the same arguments loads that plan instead of tiling again (--no-plan-file: never)\n"
             "  --check        compare the device result with the CPU path, per nonzero; exit 1 on a mismatch\n"
             "  --check-against F   compare it, per nonzero, with the nnz raw fp32 values in file F\n"
             "  --dump-out F   write the result (nnz raw fp32, sorted order) to F\n"
@@ -74,7 +76,8 @@ int main(int argc, char **argv)
     if (*endp || tx < 0) { fprintf(stderr, "sddmm: tile_size_X must be a non-negative integer\n"); return 2; }
     long ty = strtol(argv[4], &endp, 10);
     if (*endp || ty < 0) { fprintf(stderr, "sddmm: tile_size_Y must be a non-negative integer\n"); return 2; }
-    bool transpose = false, json = false, check = false, cpu_only = false, ref_order = false;
+    bool transpose = false, json = false, check = false, cpu_only = false, ref_order = false, plan_file = true;
+    bool plan_loaded = false;
     int runs = 1, cpu_threads = 0;
     long seed = 0;
     std::string check_file, dump_file;
@@ -85,6 +88,7 @@ int main(int argc, char **argv)
         if (a == "--transpose") transpose = true;
         else if (a == "--json") json = true;
         else if (a == "--check") check = true;
+        else if (a == "--no-plan-file") plan_file = false;
         else if (a == "--cpu-only") cpu_only = true;
         else if (a == "--ref-order") ref_order = true;
         else if (a == "--check-against" && i + 1 < argc) check_file = argv[++i];
@@ -152,8 +156,22 @@ int main(int argc, char **argv)
         out = cpu;
         printf("\nTilesize: X = %ld, tilesize: Y = %ld, TB: 0\n", tx, ty);
     } else {
-        CHECK(sddmm_plan_create(S, (int32_t)K, (int32_t)tx, (int32_t)ty, kernel, &plan));
+        sddmm_plan_options opt;
+        sddmm_plan_options_init(&opt);
+        opt.kernel = (int32_t)kernel; opt.tile_size_x = (int32_t)tx; opt.tile_size_y = (int32_t)ty;
+        auto plan_path = [&](const std::string &bin) {
+            return bin + ".k" + std::to_string(K) + ".x" + std::to_string(tx) + ".y" + std::to_string(ty) + "." +
+                   std::to_string(kernel) + ".plan";
+        };
+        // a plan file beside a binary input: built for this matrix, K and options, or ignored
+        if (plan_file && ends_with(input, ".bin")) {
+            if (sddmm_plan_load(plan_path(input).c_str(), S, (int32_t)K, &opt, &plan) == SDDMM_OK) plan_loaded = true;
+            else plan = nullptr;
+        }
+        if (!plan) CHECK(sddmm_plan_create_opt(S, (int32_t)K, &opt, &plan));
+        if (plan_file && !save_bin.empty() && !plan_loaded) CHECK(sddmm_plan_save(plan, plan_path(save_bin).c_str()));
         CHECK(sddmm_plan_get_info(plan, &info));
+        if (plan_loaded) fprintf(stderr, "sddmm: plan loaded from %s (%.1f ms)\n", plan_path(input).c_str(), info.plan_ms);
         printf("\nTilesize: X = %d, tilesize: Y = %d, TB: %d\n", info.tile_size_x, info.tile_size_y, info.block);
         std::vector<float> ms((size_t)runs);
         for (int r = 0; r < runs; ++r) CHECK(sddmm_gpu(plan, W.data(), H.data(), out.data(), &ms[r]));
@@ -205,10 +223,10 @@ int main(int argc, char **argv)
         printf("{\"rows\": %lld, \"cols\": %lld, \"nnz\": %lld, \"K\": %ld, \"tile_size_x\": %d, \"tile_size_y\": %d, "
                "\"kernel\": %d, \"lanes_per_nnz\": %d, \"lds_bytes\": %d, \"grid\": %d, \"block\": %d, "
                "\"n_col_tiles\": %d, \"read_ms\": %.3f, \"plan_ms\": %.3f, \"kernel_ms\": %.6f, \"gflops\": %.3f, "
-               "\"alg_gbps\": %.3f, \"cpu_ms\": %.3f, \"mismatches\": %lld, \"max_rel\": %.4g, \"checksum\": %.9g}\n",
+               "\"alg_gbps\": %.3f, \"plan_loaded\": %s, \"cpu_ms\": %.3f, \"mismatches\": %lld, \"max_rel\": %.4g, \"checksum\": %.9g}\n",
                (long long)n_rows, (long long)n_cols, (long long)nnz, K, info.tile_size_x, info.tile_size_y, info.kernel,
                info.lanes_per_nnz, info.lds_bytes, info.grid, info.block, info.n_col_tiles, read_ms, info.plan_ms,
-               (double)med, gflops, med > 0 ? balg / (med * 1e6) : 0.0, cpu_ms, diff_tot, max_rel, sum);
+               (double)med, gflops, med > 0 ? balg / (med * 1e6) : 0.0, plan_loaded ? "true" : "false", cpu_ms, diff_tot, max_rel, sum);
     }
     sddmm_plan_destroy(plan);
     sddmm_coo_destroy(S);

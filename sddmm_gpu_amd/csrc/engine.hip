@@ -4,6 +4,7 @@
 #include <chrono>
 #include <cstring>
 #include <new>
+#include <unistd.h>
 #include "internal.hpp"
 #include "kernels.hpp"
 
@@ -50,19 +51,24 @@ struct Launch {
     int32_t grid = 0, block = 0, lds = 0, k_slice = 0;
     int32_t tile_g = 0, gather_g = 8;
     int64_t nnz = 0, rows = 0, positions = 0;
+    // what the function pointers above were looked up with (they are looked up again when a saved plan is loaded)
+    int32_t fn_kind = 0;  // 1 stream kernel (row gather), 2 stream kernel with an LDS tile, 3 tile kernel, 4 panel, 5 dense
+    int32_t fn_g = 0, fn_kpl = 0, fn_exact = 0, fn_gather = 0, fn_nwaves = 0;
 };
 
 struct sddmm_plan {
     sddmm_plan_info info{};
     std::vector<Launch> launches;
-    std::vector<void *> owned;  // device allocations freed with the plan
+    struct Owned { void *p; size_t bytes; };
+    std::vector<Owned> owned;   // device allocations freed with the plan (sizes kept for sddmm_plan_save)
+    uint64_t pattern_hash = 0;  // of the CSR pattern the plan was built for (see pattern_hash_host)
     const int32_t *d_row_ptr = nullptr, *d_col = nullptr;
     float *d_val = nullptr;
     int32_t requested_kernel = 0;
     sddmm_plan_options options{};  // what the plan was built with, environment overrides applied
     ~sddmm_plan()
     {
-        for (void *p : owned) (void)hipFree(p);
+        for (const Owned &o : owned) (void)hipFree(o.p);
     }
 };
 
@@ -156,7 +162,7 @@ struct Ctx {
     int up(T **dst, const std::vector<T> &src)
     {
         int rc = upload(dst, src, &dev_bytes);
-        if (rc == SDDMM_OK && *dst) P->owned.push_back((void *)*dst);
+        if (rc == SDDMM_OK && *dst) P->owned.push_back({(void *)*dst, src.size() * sizeof(T)});
         return rc;
     }
     int need_row_ptr()
@@ -164,7 +170,7 @@ struct Ctx {
         if (P->d_row_ptr) return SDDMM_OK;
         int32_t *d = nullptr;
         HIP_TRY(hipMalloc((void **)&d, (size_t)(n_rows + 1) * 4));
-        P->owned.push_back(d);
+        P->owned.push_back({d, (size_t)(n_rows + 1) * 4});
         HIP_TRY(hipMemcpy(d, row_ptr, (size_t)(n_rows + 1) * 4, hipMemcpyHostToDevice));
         dev_bytes += (n_rows + 1) * 4;
         P->d_row_ptr = d;
@@ -210,6 +216,103 @@ void apply_env_overrides(sddmm_plan_options &o)
     i64("SDDMM_SPLIT_MIN_NNZ", o.split_min_nnz);
 }
 
+// Looks the launch's kernels up from its descriptor (fn_kind, fn_*, k_slice) and allows them its LDS size.
+int resolve_functions(Launch &L)
+{
+    L.fn = nullptr; L.pfn = nullptr; L.tfn = nullptr; L.dfn = nullptr;
+    for (auto &row : L.tfns) for (auto &f : row) f = nullptr;
+    switch (L.fn_kind) {
+    case 1:
+    case 2: {
+        const Variant v{L.fn_g, L.fn_kpl, L.fn_exact != 0};
+        L.fn = v.G ? stream_kernel(v, L.fn_kind == 2) : (L.fn_kind == 1 ? generic_kernel() : nullptr);
+        if (!L.fn) return fail(SDDMM_ERR_ARG, "plan: no stream kernel for lanes %d x %d", v.G, v.KPL);
+        if (L.lds > 0) HIP_TRY(hipFuncSetAttribute((const void *)L.fn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+        return SDDMM_OK;
+    }
+    case 3: {
+        const TileVariant tv{L.fn_g, L.fn_kpl};
+        for (int vm = 0; vm < 5; ++vm)
+            for (int ac = 0; ac < 2; ++ac) {
+                L.tfns[vm][ac] = tile_kernel(tv, vm, L.fn_gather != 0, ac != 0, L.fn_nwaves);
+                if (!L.tfns[vm][ac]) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for lanes %d x %d", tv.G, tv.KPL);
+                HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+            }
+        L.tfn = L.tfns[0][0];
+        return SDDMM_OK;
+    }
+    case 4: {
+        L.pfn = panel_kernel(pick_panel_variant(L.k_slice));
+        if (!L.pfn) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", L.k_slice);
+        if (L.lds > 0) HIP_TRY(hipFuncSetAttribute((const void *)L.pfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+        return SDDMM_OK;
+    }
+    case 5:
+        L.dfn = dense_kernel();
+        return SDDMM_OK;
+    }
+    return fail(SDDMM_ERR_FORMAT, "plan: unknown kernel descriptor %d", L.fn_kind);
+}
+
+// Order-independent 64-bit hash of a CSR pattern: the wrapping sum of a mixed word per row
+// pointer and per column index (position included), so that the host (threads) and the device
+// (atomic adds) arrive at the same value whatever order they visit the entries in.
+__host__ __device__ inline uint64_t mix64(uint64_t x)
+{
+    x ^= x >> 33; x *= 0xff51afd7ed558ccdull; x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ull; x ^= x >> 33;
+    return x;
+}
+__host__ __device__ inline uint64_t hash_row(int64_t r, int32_t v) { return mix64(((uint64_t)r << 32) ^ (uint32_t)v ^ 0x9e3779b97f4a7c15ull); }
+__host__ __device__ inline uint64_t hash_col(int64_t i, int32_t v) { return mix64(((uint64_t)i << 32) | (uint32_t)v); }
+
+uint64_t pattern_hash_host(int64_t n_rows, int64_t nnz, const int32_t *row_ptr, const int32_t *col_ind)
+{
+    std::vector<uint64_t> part((size_t)hw_threads() + 1, 0);
+    parallel_ranges(n_rows + 1, 1 << 14, [&](int64_t b, int64_t e, int t) {
+        uint64_t h = 0;
+        for (int64_t r = b; r < e; ++r) h += hash_row(r, row_ptr[r]);
+        part[(size_t)t] += h;
+    });
+    uint64_t h0 = 0;
+    for (auto &x : part) { h0 += x; x = 0; }
+    parallel_ranges(nnz, 1 << 16, [&](int64_t b, int64_t e, int t) {
+        uint64_t h = 0;
+        for (int64_t i = b; i < e; ++i) h += hash_col(i, col_ind[i]);
+        part[(size_t)t] += h;
+    });
+    for (uint64_t x : part) h0 += x;
+    return h0;
+}
+
+__global__ void pattern_hash_kernel(const int32_t *row_ptr, int64_t n_rows1, const int32_t *col_ind, int64_t nnz,
+                                    unsigned long long *acc)
+{
+    uint64_t h = 0;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x, t0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (int64_t r = t0; r < n_rows1; r += stride) h += hash_row(r, row_ptr[r]);
+    for (int64_t i = t0; i < nnz; i += stride) h += hash_col(i, col_ind[i]);
+    // one atomic per wave: the lanes' sums are added up first
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t lo = __shfl_xor((uint32_t)h, off), hi = __shfl_xor((uint32_t)(h >> 32), off);
+        h += ((uint64_t)hi << 32) | lo;
+    }
+    if ((threadIdx.x & 63) == 0) atomicAdd(acc, (unsigned long long)h);
+}
+
+int pattern_hash_device(int64_t n_rows, int64_t nnz, const int32_t *d_row_ptr, const int32_t *d_col_ind, uint64_t *out)
+{
+    unsigned long long *d_acc = nullptr;
+    HIP_TRY(hipMalloc((void **)&d_acc, 8));
+    struct Free { void *p; ~Free() { (void)hipFree(p); } } fr{d_acc};
+    HIP_TRY(hipMemset(d_acc, 0, 8));
+    hipLaunchKernelGGL(pattern_hash_kernel, dim3(2048), dim3(256), 0, nullptr, d_row_ptr, n_rows + 1, d_col_ind, nnz, d_acc);
+    HIP_TRY(hipGetLastError());
+    unsigned long long h = 0;
+    HIP_TRY(hipMemcpy(&h, d_acc, 8, hipMemcpyDeviceToHost));
+    *out = (uint64_t)h;
+    return SDDMM_OK;
+}
+
 int64_t list_nnz(const Ctx &c, const std::vector<int32_t> &rows)
 {
     int64_t n = 0;
@@ -230,8 +333,8 @@ int add_row_gather(Ctx &c, const std::vector<int32_t> &rows, bool all_rows)
     if (n == 0) return SDDMM_OK;
     const bool vec4 = c.K % 4 == 0;
     Variant var = vec4 ? pick_variant(c.K, false) : Variant{0, 0, false};
-    L.fn = var.G ? stream_kernel(var, false) : generic_kernel();
-    if (!L.fn) return fail(SDDMM_ERR_ARG, "plan: no row-gather kernel for K = %d", c.K);
+    L.fn_kind = 1; L.fn_g = var.G; L.fn_kpl = var.KPL; L.fn_exact = var.exact;
+    if (int rc = resolve_functions(L)) return rc;
     std::vector<int32_t> seg_end(rows.size()), perm;
     int64_t acc = 0;
     for (size_t i = 0; i < rows.size(); ++i) {
@@ -284,8 +387,8 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     L.kind = SDDMM_KERNEL_LDS_TILE;
     L.rows = (int64_t)rows.size();
     Variant var = pick_variant(c.K, true);
-    L.fn = var.G ? stream_kernel(var, true) : nullptr;
-    if (!L.fn) return fail(SDDMM_ERR_ARG, "plan: no LDS-tile kernel for K = %d", c.K);
+    if (!var.G) return fail(SDDMM_ERR_ARG, "plan: no LDS-tile kernel for K = %d", c.K);
+    L.fn_kind = 2; L.fn_g = var.G; L.fn_kpl = var.KPL; L.fn_exact = var.exact;
     sddmm_tiling T;
     if (int rc = build_tiling(c.n_rows, c.n_cols, c.nnz, c.row_ptr, c.col_ind, x, y, T, all_rows ? nullptr : rows.data(),
                               (int64_t)rows.size()))
@@ -352,7 +455,7 @@ int add_lds_tile(Ctx &c, const std::vector<int32_t> &rows, bool all_rows, int32_
     L.block = kLdsBlock;
     L.lds = (int32_t)((int64_t)x * c.K * 4);
     L.k_slice = c.K;
-    HIP_TRY(hipFuncSetAttribute((const void *)L.fn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (int rc = resolve_functions(L)) return rc;
     if (I) {
         I->tile_size_x = x; I->tile_size_y = y; I->n_col_tiles = T.n_tiles;
         I->n_row_panels = (int32_t)((T.max_active_rows + y - 1) / y);
@@ -379,10 +482,8 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // 12 waves per workgroup measured 2-5 % faster than 16 on slices of 64 and 128, slower on 32
     int nwaves = gather ? 4 : (int)(c.opt.tile_waves > 0 ? c.opt.tile_waves : (ks >= 64 ? 12 : 16));
     if (!gather && nwaves != 12) nwaves = 16;
-    L.tfn = tv.G ? tile_kernel(tv, 0, gather, false, nwaves) : nullptr;
-    if (!L.tfn) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
-    for (int vm = 0; vm < 5; ++vm)
-        for (int ac = 0; ac < 2; ++ac) L.tfns[vm][ac] = tile_kernel(tv, vm, gather, ac != 0, nwaves);
+    if (!tv.G || !tile_kernel(tv, 0, gather, false, nwaves)) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
+    L.fn_kind = 3; L.fn_g = tv.G; L.fn_kpl = tv.KPL; L.fn_gather = gather; L.fn_nwaves = nwaves;
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
     if (L.nnz == 0) return SDDMM_OK;
@@ -775,9 +876,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
     L.k_slice = ks;
     if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
-    for (int vm = 0; vm < 5; ++vm)
-        for (int ac = 0; ac < 2; ++ac)
-            HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (int rc = resolve_functions(L)) return rc;
     if (I) {
         I->tile_size_x = x; I->tile_size_y = panel_rows; I->n_col_tiles = n_tiles_all;
         I->n_row_panels = n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
@@ -794,7 +893,8 @@ int add_dense(Ctx &c, const DenseBlocks &D, const float *vals_all)
 {
     Launch L;
     L.kind = SDDMM_KERNEL_DENSE_BLOCK;
-    L.dfn = dense_kernel();
+    L.fn_kind = 5;
+    if (int rc = resolve_functions(L)) return rc;
     L.nnz = D.n_dense;
     const int64_t n_tiles = (int64_t)D.tile_rb.size();
     // Schedule: workgroup b runs on die b % 8 (each die has its own L2) and takes slots b, b + grid, ...
@@ -872,8 +972,8 @@ int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, 
     L.nnz = list_nnz(c, rows);
     if (L.nnz == 0) return SDDMM_OK;
     const PanelVariant pv = pick_panel_variant(ks);
-    L.pfn = panel_kernel(pv);
-    if (!L.pfn) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", ks);
+    if (!panel_kernel(pv)) return fail(SDDMM_ERR_ARG, "plan: no panel kernel for K slice %d", ks);
+    L.fn_kind = 4;
     const int32_t fit = kLdsMaxBytes / (ks * 4);
     int32_t x = tile_x > 0 ? std::min(tile_x, fit) : fit;
     x = (int32_t)std::min<int64_t>(x, std::max<int64_t>(c.n_cols, 1));
@@ -925,7 +1025,7 @@ int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, 
     L.block = pv.NWAVES * 64;
     L.lds = x * ks * 4;
     L.k_slice = ks;
-    HIP_TRY(hipFuncSetAttribute((const void *)L.pfn, hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+    if (int rc = resolve_functions(L)) return rc;
     if (I) {
         I->tile_size_x = x; I->tile_size_y = rows_per_panel; I->k_slice = ks;
         I->n_col_tiles = (int32_t)((c.n_cols + x - 1) / x); I->n_row_panels = (int32_t)n_panels;
@@ -966,6 +1066,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     I.n_rows = n_rows; I.n_cols = n_cols; I.nnz = nnz; I.K = K; I.k_slice = K;
     count_touched(n_rows, n_cols, nnz, row_ptr_all, col_ind_all, &I.rows_touched, &I.cols_touched);
     P->requested_kernel = want;
+    P->pattern_hash = pattern_hash_host(n_rows, nnz, row_ptr_all, col_ind_all);
     // what the gathering kernels work on: S itself, or what is left of it once the dense blocks are cut out
     const int32_t *row_ptr = row_ptr_all, *col_ind = col_ind_all;
     int64_t nnz_part = nnz;
@@ -982,14 +1083,14 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     } else if (nnz) {
         int32_t *d = nullptr;
         HIP_TRY(hipMalloc((void **)&d, (size_t)nnz * 4));
-        P->owned.push_back(d);
+        P->owned.push_back({d, (size_t)nnz * 4});
         HIP_TRY(hipMemcpy(d, col_ind_all, (size_t)nnz * 4, hipMemcpyHostToDevice));
         c.dev_bytes += nnz * 4;
         P->d_col = d;
     }
     if (vals && nnz) {
         HIP_TRY(hipMalloc((void **)&P->d_val, (size_t)nnz * 4));
-        P->owned.push_back(P->d_val);
+        P->owned.push_back({P->d_val, (size_t)nnz * 4});
         HIP_TRY(hipMemcpy(P->d_val, vals, (size_t)nnz * 4, hipMemcpyHostToDevice));
         c.dev_bytes += nnz * 4;
     }
@@ -1339,7 +1440,7 @@ int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
     if (!d_val) return fail(SDDMM_ERR_ARG, "sddmm_plan_set_values: d_val is NULL");
     if (!plan->d_val) {
         HIP_TRY(hipMalloc((void **)&plan->d_val, (size_t)nnz * 4));
-        plan->owned.push_back(plan->d_val);
+        plan->owned.push_back({plan->d_val, (size_t)nnz * 4});
         plan->info.device_bytes += nnz * 4;
     }
     HIP_TRY(hipMemcpyAsync(plan->d_val, d_val, (size_t)nnz * 4, hipMemcpyDeviceToDevice, (hipStream_t)stream));
@@ -1347,13 +1448,309 @@ int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
         if (!L.perm || L.positions <= 0) continue;  // walks S in sorted order: reads d_val directly
         if (!L.sval) {
             HIP_TRY(hipMalloc((void **)&L.sval, ((size_t)L.positions + kStreamSlack) * 4));  // (see add_tile)
-            plan->owned.push_back(L.sval);
+            plan->owned.push_back({L.sval, ((size_t)L.positions + kStreamSlack) * 4});
             plan->info.device_bytes += L.positions * 4;
         }
         launch_gather_values(L.perm, plan->d_val, L.sval, L.positions, stream);
     }
     HIP_TRY(hipGetLastError());
     return SDDMM_OK;
+}
+
+// ---- plan files -------------------------------------------------------------
+// A plan file is the plan's device arrays and launch descriptors under a header with the key it
+// was built for.  Device pointers are stored as (allocation number + 1) << 44 | byte offset.
+namespace {
+
+struct PlanFileHeader {
+    char magic[8];
+    uint32_t version, sizeof_launch, sizeof_info, sizeof_options;
+    int64_t n_rows, n_cols, nnz;
+    int32_t K, requested_kernel;
+    uint64_t pattern_hash;
+    uint64_t n_allocs, n_launches;
+    uint64_t code_row_ptr, code_col, code_val;
+    char build[40];
+};
+constexpr char kPlanMagic[8] = {'S', 'D', 'D', 'M', 'M', 'P', 'L', 'N'};
+constexpr uint32_t kPlanVersion = 2;
+constexpr uint64_t kBorrowedRowPtr = (1ull << 63) | 1, kBorrowedCol = (1ull << 63) | 2;
+
+// every pointer of a launch that refers to memory the plan owns
+void launch_pointer_fields(Launch &L, std::vector<void *> &fields)
+{
+    fields = {&L.ka.perm, &L.ka.scol, &L.ka.seg_row, &L.ka.batch_seg, &L.ka.batch_mask, &L.ka.items,
+            &L.ta.perm, &L.ta.scol, &L.ta.grow, &L.ta.scol16, &L.ta.pbase, &L.ta.btype, &L.ta.sink, &L.ta.unit_ptr,
+            &L.ta.unit_tile, &L.ta.items,
+            &L.pa.slot_row, &L.pa.panel_tiles,
+            &L.da.slot_rows, &L.da.slot_cols, &L.da.slot_range, &L.da.nz_p, &L.da.nz_rc,
+            &L.sval, &L.perm};
+}
+
+bool encode_pointer(const sddmm_plan *P, const void *p, uint64_t *code)
+{
+    *code = 0;
+    if (!p) return true;
+    for (size_t i = 0; i < P->owned.size(); ++i) {
+        const char *b = (const char *)P->owned[i].p;
+        if ((const char *)p >= b && (const char *)p < b + P->owned[i].bytes) {
+            *code = ((uint64_t)(i + 1) << 44) | (uint64_t)((const char *)p - b);
+            return true;
+        }
+    }
+    return false;
+}
+
+bool decode_pointer(const sddmm_plan *P, uint64_t code, void **p)
+{
+    *p = nullptr;
+    if (!code) return true;
+    const uint64_t i = (code >> 44), off = code & ((1ull << 44) - 1);
+    if (i < 1 || i > P->owned.size() || off >= P->owned[i - 1].bytes) return false;
+    *p = (char *)P->owned[i - 1].p + off;
+    return true;
+}
+
+bool same_options(const sddmm_plan_options &a, const sddmm_plan_options &b)
+{
+    sddmm_plan_options x = a, y = b;
+    x.ignore_env = y.ignore_env = 0;  // how the values got there is not part of the key
+    if (x.tile_lanes < 0) x.tile_lanes = 0;
+    if (y.tile_lanes < 0) y.tile_lanes = 0;
+    return memcmp(&x, &y, sizeof x) == 0;
+}
+
+struct FileCloser { FILE *f; ~FileCloser() { if (f) fclose(f); } };
+
+int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz, int32_t K, const sddmm_plan_options *opt_in,
+                   const uint64_t *want_hash, const int32_t *d_row_ptr, const int32_t *d_col_ind, sddmm_plan **out)
+{
+    auto t0 = std::chrono::steady_clock::now();
+    if (int rc = device_ok()) return rc;
+    FILE *f = fopen(path, "rb");
+    if (!f) return fail(SDDMM_ERR_IO, "sddmm_plan_load: cannot open %s", path);
+    FileCloser fc{f};
+    PlanFileHeader h;
+    if (fread(&h, sizeof h, 1, f) != 1 || memcmp(h.magic, kPlanMagic, 8) != 0)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is not a plan file", path);
+    h.build[sizeof h.build - 1] = 0;
+    if (h.version != kPlanVersion || h.sizeof_launch != sizeof(Launch) || h.sizeof_info != sizeof(sddmm_plan_info) ||
+        h.sizeof_options != sizeof(sddmm_plan_options) || strncmp(h.build, sddmm_version(), sizeof h.build - 1) != 0)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s was written by another build of the library (%s)", path, h.build);
+    if (h.n_rows != n_rows || h.n_cols != n_cols || h.nnz != nnz || h.K != K)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s holds a plan for %lld x %lld, nnz %lld, K %d, not for %lld x %lld, nnz %lld, K %d",
+                    path, (long long)h.n_rows, (long long)h.n_cols, (long long)h.nnz, h.K, (long long)n_rows, (long long)n_cols,
+                    (long long)nnz, K);
+    if (want_hash && *want_hash != h.pattern_hash)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s was built for another sparsity pattern", path);
+    if (h.n_allocs > (1u << 20) || h.n_launches > (1u << 16)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged", path);
+    sddmm_plan *P = new (std::nothrow) sddmm_plan;
+    if (!P) return fail(SDDMM_ERR_NOMEM, "sddmm_plan_load: out of memory");
+    struct Guard { sddmm_plan *p; ~Guard() { delete p; } } guard{P};
+    if (fread(&P->info, sizeof P->info, 1, f) != 1 || fread(&P->options, sizeof P->options, 1, f) != 1)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is cut short", path);
+    if (opt_in) {
+        sddmm_plan_options want = *opt_in;
+        apply_env_overrides(want);
+        if (!same_options(want, P->options))
+            return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s was built with other plan options", path);
+    }
+    std::vector<uint64_t> sizes((size_t)h.n_allocs);
+    if (h.n_allocs && fread(sizes.data(), 8, sizes.size(), f) != sizes.size())
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is cut short", path);
+    P->launches.resize((size_t)h.n_launches);
+    if (h.n_launches && fread((void *)P->launches.data(), sizeof(Launch), P->launches.size(), f) != P->launches.size())
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is cut short", path);
+    // The arrays: pieces of 16 MiB are read (pread) by a few threads, each into its own pair of pinned
+    // staging buffers, and copied to the device on the thread's own stream as they arrive.
+    constexpr size_t kPiece = (size_t)16 << 20;
+    const long data_at = ftell(f);
+    if (data_at < 0) return fail(SDDMM_ERR_IO, "sddmm_plan_load: cannot seek in %s", path);
+    struct Piece { void *dst; uint64_t file_off; size_t n; };
+    std::vector<Piece> pieces;
+    int64_t total = 0;
+    {
+        uint64_t at = (uint64_t)data_at;
+        for (uint64_t bytes : sizes) {
+            if (bytes == 0 || bytes > ((uint64_t)1 << 40)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged", path);
+            void *d = nullptr;
+            HIP_TRY(hipMalloc(&d, bytes));
+            P->owned.push_back({d, (size_t)bytes});
+            total += (int64_t)bytes;
+            for (uint64_t off = 0; off < bytes; off += kPiece)
+                pieces.push_back({(char *)d + off, at + off, (size_t)std::min<uint64_t>(kPiece, bytes - off)});
+            at += bytes;
+        }
+    }
+    const int n_readers = (int)std::max<size_t>(1, std::min<size_t>({(size_t)8, (size_t)hw_threads(), pieces.size()}));
+    std::vector<int> reader_rc((size_t)n_readers, 0);  // 0 ok, 1 short read, 2 HIP error
+    const int fd = fileno(f);
+    {
+        std::vector<std::thread> th;
+        for (int t = 0; t < n_readers; ++t)
+            th.emplace_back([&, t] {
+                void *stage[2] = {nullptr, nullptr};
+                hipEvent_t done[2] = {nullptr, nullptr};
+                hipStream_t st = nullptr;
+                bool ok = hipStreamCreate(&st) == hipSuccess;
+                for (int i = 0; i < 2 && ok; ++i)
+                    ok = hipHostMalloc(&stage[i], kPiece, hipHostMallocDefault) == hipSuccess && hipEventCreate(&done[i]) == hipSuccess;
+                int turn = 0;
+                for (size_t k = (size_t)t; ok && k < pieces.size(); k += (size_t)n_readers, turn ^= 1) {
+                    const Piece &pc = pieces[k];
+                    if (hipEventSynchronize(done[turn]) != hipSuccess) { ok = false; break; }  // (never recorded: complete)
+                    size_t got = 0;
+                    while (got < pc.n) {
+                        const ssize_t r = pread(fd, (char *)stage[turn] + got, pc.n - got, (off_t)(pc.file_off + got));
+                        if (r <= 0) break;
+                        got += (size_t)r;
+                    }
+                    if (got != pc.n) { reader_rc[(size_t)t] = 1; break; }
+                    ok = hipMemcpyAsync(pc.dst, stage[turn], pc.n, hipMemcpyHostToDevice, st) == hipSuccess &&
+                         hipEventRecord(done[turn], st) == hipSuccess;
+                }
+                if (st) ok = (hipStreamSynchronize(st) == hipSuccess) && ok;
+                if (!ok && !reader_rc[(size_t)t]) reader_rc[(size_t)t] = 2;
+                for (int i = 0; i < 2; ++i) { if (stage[i]) (void)hipHostFree(stage[i]); if (done[i]) (void)hipEventDestroy(done[i]); }
+                if (st) (void)hipStreamDestroy(st);
+            });
+        for (auto &x : th) x.join();
+    }
+    for (int rc : reader_rc) {
+        if (rc == 1) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is cut short", path);
+        if (rc == 2) return fail(SDDMM_ERR_HIP, "sddmm_plan_load: copying %s to the device failed", path);
+    }
+    HIP_TRY(hipDeviceSynchronize());
+    // pointers
+    void *q = nullptr;
+    std::vector<void *> fields;
+    for (Launch &L : P->launches) {
+        launch_pointer_fields(L, fields);
+        for (void *field : fields) {
+            uint64_t code;
+            memcpy(&code, field, 8);
+            if (!decode_pointer(P, code, &q)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged (bad reference)", path);
+            memcpy(field, &q, 8);
+        }
+        L.ka.col_ind = nullptr; L.ka.val = nullptr; L.ka.W = L.ka.H = nullptr; L.ka.out = nullptr; L.ka.sval = nullptr;
+        L.ka.row_ptr = nullptr; L.ka.batch_row = nullptr;
+        L.ta.sval = nullptr; L.ta.val = nullptr; L.ta.W = L.ta.H = nullptr; L.ta.out = nullptr;
+        L.pa.row_ptr = nullptr; L.pa.col_ind = nullptr; L.pa.val = nullptr; L.pa.W = L.pa.H = nullptr; L.pa.out = nullptr;
+        L.da.nz_val = nullptr; L.da.val = nullptr; L.da.W = L.da.H = nullptr; L.da.out = nullptr;
+        if (int rc = resolve_functions(L)) return rc;
+    }
+    auto place = [&](uint64_t code, const int32_t *borrowed, uint64_t marker, const void **dst) -> bool {
+        if (code == marker) { *dst = borrowed; return borrowed != nullptr; }
+        void *x = nullptr;
+        if (!decode_pointer(P, code, &x)) return false;
+        *dst = x;
+        return true;
+    };
+    const void *rp = nullptr, *ci = nullptr;
+    if (!place(h.code_row_ptr, d_row_ptr, kBorrowedRowPtr, &rp) || !place(h.code_col, d_col_ind, kBorrowedCol, &ci))
+        return fail(SDDMM_ERR_ARG, "sddmm_plan_load: %s holds a plan over a device-resident pattern: pass d_row_ptr and d_col_ind "
+                                   "(sddmm_plan_load_device)", path);
+    P->d_row_ptr = (const int32_t *)rp; P->d_col = (const int32_t *)ci;
+    if (!decode_pointer(P, h.code_val, &q)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged (bad reference)", path);
+    P->d_val = (float *)q;
+    P->requested_kernel = h.requested_kernel;
+    P->pattern_hash = h.pattern_hash;
+    P->info.device_bytes = total;
+    P->info.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    guard.p = nullptr;
+    *out = P;
+    return SDDMM_OK;
+}
+
+}  // namespace
+
+int sddmm_plan_save(const sddmm_plan *plan, const char *path)
+{
+    if (!plan || !path) return fail(SDDMM_ERR_ARG, "sddmm_plan_save: NULL argument");
+    try {
+        PlanFileHeader h;
+        memset(&h, 0, sizeof h);
+        memcpy(h.magic, kPlanMagic, 8);
+        h.version = kPlanVersion; h.sizeof_launch = sizeof(Launch); h.sizeof_info = sizeof(sddmm_plan_info);
+        h.sizeof_options = sizeof(sddmm_plan_options);
+        h.n_rows = plan->info.n_rows; h.n_cols = plan->info.n_cols; h.nnz = plan->info.nnz; h.K = plan->info.K;
+        h.requested_kernel = plan->requested_kernel; h.pattern_hash = plan->pattern_hash;
+        h.n_allocs = plan->owned.size(); h.n_launches = plan->launches.size();
+        strncpy(h.build, sddmm_version(), sizeof h.build - 1);
+        if (!encode_pointer(plan, plan->d_row_ptr, &h.code_row_ptr)) h.code_row_ptr = kBorrowedRowPtr;
+        if (!encode_pointer(plan, plan->d_col, &h.code_col)) h.code_col = kBorrowedCol;
+        if (!encode_pointer(plan, plan->d_val, &h.code_val)) return fail(SDDMM_ERR_ARG, "sddmm_plan_save: values outside the plan's memory");
+        std::vector<Launch> ls(plan->launches);
+        std::vector<void *> fields;
+        for (Launch &L : ls) {
+            launch_pointer_fields(L, fields);
+            for (void *field : fields) {
+                const void *p;
+                memcpy(&p, field, 8);
+                uint64_t code;
+                if (!encode_pointer(plan, p, &code)) return fail(SDDMM_ERR_ARG, "sddmm_plan_save: a launch refers to memory outside the plan");
+                memcpy(field, &code, 8);
+            }
+            L.fn = nullptr; L.pfn = nullptr; L.tfn = nullptr; L.dfn = nullptr;
+            for (auto &row : L.tfns) for (auto &fp : row) fp = nullptr;
+        }
+        HIP_TRY(hipDeviceSynchronize());  // a set_values still in flight has to land first
+        FILE *f = fopen(path, "wb");
+        if (!f) return fail(SDDMM_ERR_IO, "sddmm_plan_save: cannot create %s", path);
+        FileCloser fc{f};
+        bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(&plan->info, sizeof plan->info, 1, f) == 1 &&
+                  fwrite(&plan->options, sizeof plan->options, 1, f) == 1;
+        std::vector<uint64_t> sizes;
+        for (const auto &o : plan->owned) sizes.push_back((uint64_t)o.bytes);
+        ok = ok && (sizes.empty() || fwrite(sizes.data(), 8, sizes.size(), f) == sizes.size());
+        ok = ok && (ls.empty() || fwrite((const void *)ls.data(), sizeof(Launch), ls.size(), f) == ls.size());
+        std::vector<char> buf;
+        for (const auto &o : plan->owned) {
+            constexpr size_t kPiece = (size_t)64 << 20;
+            for (size_t off = 0; ok && off < o.bytes; off += kPiece) {
+                const size_t n = std::min(kPiece, o.bytes - off);
+                buf.resize(n);
+                HIP_TRY(hipMemcpy(buf.data(), (const char *)o.p + off, n, hipMemcpyDeviceToHost));
+                ok = fwrite(buf.data(), 1, n, f) == n;
+            }
+        }
+        if (!ok || fflush(f) != 0) return fail(SDDMM_ERR_IO, "sddmm_plan_save: write to %s failed", path);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_save: %s", e.what());
+    }
+    return SDDMM_OK;
+}
+
+int sddmm_plan_load(const char *path, const sddmm_coo *S, int32_t K, const sddmm_plan_options *opt, sddmm_plan **out)
+{
+    if (!path || !S || !out) return fail(SDDMM_ERR_ARG, "sddmm_plan_load: NULL argument");
+    *out = nullptr;
+    if (S->sorted != 1) return fail(SDDMM_ERR_UNSORTED, "sddmm_plan_load: matrix is not (row, col)-sorted");
+    try {
+        std::vector<int32_t> rp;
+        build_row_ptr(*S, rp);
+        const uint64_t hash = pattern_hash_host(S->n_rows, S->nnz, rp.data(), S->cols.data());
+        return load_plan_file(path, S->n_rows, S->n_cols, S->nnz, K, opt, &hash, nullptr, nullptr, out);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_load: %s", e.what());
+    }
+}
+
+int sddmm_plan_load_device(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                           const int32_t *d_col_ind, int32_t K, const sddmm_plan_options *opt, sddmm_plan **out)
+{
+    if (!path || !out) return fail(SDDMM_ERR_ARG, "sddmm_plan_load_device: NULL argument");
+    *out = nullptr;
+    if (n_rows < 0 || n_cols < 0 || nnz < 0 || !d_row_ptr || (nnz > 0 && !d_col_ind))
+        return fail(SDDMM_ERR_ARG, "sddmm_plan_load_device: bad sizes or NULL arrays");
+    if (int rc = device_ok()) return rc;
+    try {
+        uint64_t hash = 0;
+        if (int rc = pattern_hash_device(n_rows, nnz, d_row_ptr, d_col_ind, &hash)) return rc;
+        return load_plan_file(path, n_rows, n_cols, nnz, K, opt, &hash, d_row_ptr, d_col_ind, out);
+    } catch (const std::exception &e) {
+        return fail(SDDMM_ERR_NOMEM, "sddmm_plan_load_device: %s", e.what());
+    }
 }
 
 int sddmm_plan_launch_count(const sddmm_plan *plan, int32_t *n)
