@@ -307,6 +307,29 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
 int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
                            float *d_out, int32_t epilogue, void *stream);
 
+/* The forms that surround an SDDMM where it is used as sparse attention or
+ * in graph networks -- "SDDMM ... is a core of many machine learning
+ * algorithms" (README.md:1); the reference itself stops at the sampled product.
+ *
+ * sddmm_execute_softmax: sddmm_execute followed, on the same stream, by the
+ * row-wise softmax of the results in place:
+ *   out[p] = exp(s_p - m_r) / sum_{q in row r} exp(s_q - m_r),  s = val .* (W H^T) on S's pattern,
+ * m_r the row's largest s.  One extra pass over out (the row totals must be known
+ * before any entry can be normalised); rows up to 512 entries are read once.
+ * sddmm_row_softmax: the same pass on its own, over any CSR pattern in device
+ * memory (d_out may be d_x).
+ * sddmm_spmm_csr: Y[r, 0:K] = sum over row r's entries p of x[p] * H[col_p, 0:K]
+ * (d_Y: n_rows*K fp32, overwritten; rows without entries become 0), the product
+ * that consumes the attention weights.  Rows that straddle the 256-entry chunks
+ * the waves work in are completed with fp32 atomic adds, so their last bits can
+ * differ from run to run.                                                    */
+int sddmm_execute_softmax(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                          float *d_out, void *stream);
+int sddmm_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream);
+int sddmm_spmm_csr(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
+                   const int32_t *d_col_ind, const float *d_x, int32_t K, const float *d_H, float *d_Y,
+                   void *stream);
+
 /* The same execution with an event after every launch-list entry: fills one
  * profile per entry (sddmm_plan_launch_count of them) with its wall time on
  * the device, then returns (synchronises on the last event).  No counterpart

@@ -111,6 +111,26 @@ def sddmm_f64(row_ind, col_ind, val, W, H):
     return out, absp
 
 
+def row_softmax(row_ptr, x):
+    """Row-wise softmax over the stored entries (accumulated in fp64, rounded once)."""
+    row_ptr, x = _i32(row_ptr), _f32(x)
+    out = np.zeros(len(x), np.float32)
+    lib().oracle_row_softmax(c_int64(len(row_ptr) - 1), _p(row_ptr), _p(x), _p(out))
+    return out
+
+
+def spmm_csr(row_ptr, col_ind, x, H, with_abs=False):
+    """Y[r,:] = sum_p x[p] * H[col_p,:], sequential fp32; with_abs: also sum |x*h| in fp64."""
+    row_ptr, col_ind, x, H = _i32(row_ptr), _i32(col_ind), _f32(x), _f32(H)
+    n_rows = len(row_ptr) - 1
+    k = H.shape[1]
+    Y = np.empty((n_rows, k), np.float32)
+    absy = np.empty((n_rows, k), np.float64) if with_abs else None
+    lib().oracle_spmm_csr(c_int64(n_rows), _p(row_ptr), _p(col_ind), _p(x), c_int32(k), _p(H), _p(Y),
+                          _p(absy) if with_abs else None)
+    return (Y, absy) if with_abs else Y
+
+
 def make_csr(rows, n_rows):
     rows = _i32(rows)
     row_ptr = np.zeros(n_rows + 2, np.int32)

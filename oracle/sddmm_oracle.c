@@ -24,6 +24,14 @@
  *                            and oracle/_ref
  *   oracle_transpose_sort    scipy coo->csr of the transposed triples
  *   oracle_parse_mtx         hand-written files with known contents
+ *   oracle_row_softmax,
+ *   oracle_spmm_csr          the two forms that surround an SDDMM in its machine-
+ *                            learning uses (reference README.md:1); the reference
+ *                            has no code for them, so they restate the textbook
+ *                            definitions and are pinned by closed forms (equal
+ *                            logits -> 1/row length, rows sum to 1, shift
+ *                            invariance; one-hot H -> column pick), by
+ *                            scipy.sparse (csr @ H) and by fp64 brute force
  */
 #define _XOPEN_SOURCE 600
 #include <stdint.h>
@@ -31,6 +39,7 @@
 #include <string.h>
 #include <stdio.h>
 #include <ctype.h>
+#include <math.h>
 #ifdef _OPENMP
 #include <omp.h>
 #endif
@@ -341,4 +350,46 @@ int oracle_parse_mtx(const char *path, int64_t *n_rows, int64_t *n_cols,
     }
     fclose(f);
     return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Row-wise softmax over the stored entries of a CSR matrix:
+ * out[p] = exp(x[p] - max_r) / sum_{q in row r} exp(x[q] - max_r).
+ * The reference has no such code (README.md:1 names the use); this is the
+ * definition, accumulated in double and rounded once, so that it can serve as
+ * the exact value an fp32 implementation approximates.                   */
+void oracle_row_softmax(int64_t n_rows, const int32_t *row_ptr, const float *x, float *out)
+{
+    #pragma omp parallel for schedule(dynamic, 256)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        const int64_t b = row_ptr[r], e = row_ptr[r + 1];
+        if (e <= b) continue;
+        float mx = x[b];
+        for (int64_t p = b + 1; p < e; ++p) mx = x[p] > mx ? x[p] : mx;
+        double sum = 0.0;
+        for (int64_t p = b; p < e; ++p) sum += exp((double)x[p] - (double)mx);
+        for (int64_t p = b; p < e; ++p) out[p] = (float)(exp((double)x[p] - (double)mx) / sum);
+    }
+}
+
+/* Y[r, 0:k] = sum over the row's entries p (in order) of x[p] * H[col_p, 0:k], fp32, sequential:
+ * the sparse-times-dense product that follows an SDDMM in attention-like uses.  absy (may be NULL)
+ * receives sum |x[p] * H[col_p, t]| in double, the conditioning term for error bounds.            */
+void oracle_spmm_csr(int64_t n_rows, const int32_t *row_ptr, const int32_t *col_ind, const float *x, int32_t k,
+                     const float *H, float *Y, double *absy)
+{
+    #pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t r = 0; r < n_rows; ++r) {
+        float *y = Y + r * k;
+        for (int32_t t = 0; t < k; ++t) y[t] = 0.0f;
+        if (absy) for (int32_t t = 0; t < k; ++t) absy[r * k + t] = 0.0;
+        for (int64_t p = row_ptr[r]; p < row_ptr[r + 1]; ++p) {
+            const float *h = H + (int64_t)col_ind[p] * k;
+            for (int32_t t = 0; t < k; ++t) {
+                float prod = x[p] * h[t];
+                y[t] = y[t] + prod;
+                if (absy) absy[r * k + t] += fabs((double)x[p] * (double)h[t]);
+            }
+        }
+    }
 }

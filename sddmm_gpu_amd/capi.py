@@ -111,6 +111,9 @@ SIGNATURES = {
     "sddmm_plan_destroy": (None, [c_void_p]),
     "sddmm_execute": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sddmm_execute_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
+    "sddmm_execute_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sddmm_row_softmax": (c_int, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sddmm_spmm_csr": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
     "sddmm_execute_profiled": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(LaunchProfile), c_int32]),
     "sddmm_gpu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, POINTER(c_float)]),
@@ -330,6 +333,10 @@ class Plan:
         check(lib().sddmm_execute_epilogue(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
                                            c_int32(epilogue), c_void_p(stream or None)))
 
+    def execute_softmax(self, d_val, d_W, d_H, d_out, stream=0):
+        check(lib().sddmm_execute_softmax(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
+                                          c_void_p(stream or None)))
+
     def execute_profiled(self, d_val, d_W, d_H, d_out, stream=0):
         n = c_int32()
         check(lib().sddmm_plan_launch_count(self.h, byref(n)))
@@ -372,6 +379,15 @@ def csr_noalloc(n_rows, n_cols, nnz, d_row_ptr, d_col_ind, d_val, K, d_W, d_H, d
     """Plan-free SDDMM over a device CSR that allocates nothing (sddmm_csr_noalloc)."""
     check(lib().sddmm_csr_noalloc(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind), c_void_p(d_val or None), K,
                                   c_void_p(d_W), c_void_p(d_H), c_void_p(d_out), c_void_p(stream or None)))
+
+
+def row_softmax(n_rows, d_row_ptr, d_x, d_out, stream=0):
+    check(lib().sddmm_row_softmax(n_rows, c_void_p(d_row_ptr), c_void_p(d_x), c_void_p(d_out), c_void_p(stream or None)))
+
+
+def spmm_csr(n_rows, n_cols, nnz, d_row_ptr, d_col_ind, d_x, K, d_H, d_Y, stream=0):
+    check(lib().sddmm_spmm_csr(n_rows, n_cols, nnz, c_void_p(d_row_ptr), c_void_p(d_col_ind or None), c_void_p(d_x or None), K,
+                               c_void_p(d_H or None), c_void_p(d_Y), c_void_p(stream or None)))
 
 
 def copy_probe(d_src, d_dst, n_bytes, stream=0):

@@ -1242,6 +1242,10 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         } else if (int rc = add_row_gather(c, ne, true)) return rc;
         I.kernel = SDDMM_KERNEL_ROW_GATHER; I.class_nnz[2] = nnz; I.class_rows[2] = (int64_t)ne.size();
     }
+    // the row pointers stay with the plan (the row-wise softmax epilogue walks S row by row)
+    c.row_ptr = row_ptr_all;
+    if (nnz > 0)
+        if (int rc = c.need_row_ptr()) return rc;
     if (!P->launches.empty() && I.grid == 0) { I.grid = P->launches[0].grid; I.block = P->launches[0].block; I.lds_bytes = P->launches[0].lds; }
     I.n_launches = 0;
     for (const Launch &L : P->launches) I.n_launches += (L.k_slice > 0 && L.k_slice < K) ? K / L.k_slice : 1;
@@ -1430,6 +1434,15 @@ int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const flo
     for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream, epilogue);
     HIP_TRY(hipGetLastError());
     return SDDMM_OK;
+}
+
+int sddmm_execute_softmax(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H, float *d_out,
+                          void *stream)
+{
+    if (int rc = sddmm_execute(plan, d_val, d_W, d_H, d_out, stream)) return rc;
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    if (!plan->d_row_ptr) return fail(SDDMM_ERR_ARG, "sddmm_execute_softmax: the plan holds no row pointers");
+    return launch_row_softmax(plan->info.n_rows, plan->d_row_ptr, d_out, d_out, stream);
 }
 
 int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)

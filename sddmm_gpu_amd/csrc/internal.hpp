@@ -47,6 +47,9 @@ void parallel_ranges(int64_t n, int64_t grain,
 // take in turn from a shared counter (for work of uneven cost per index).
 void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t, int64_t, int)> &f);
 
+// out[p] = softmax over the entries of p's row of x (out may be x), on `stream` (a hipStream_t)
+int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream);
+
 bool check_sorted(const sddmm_coo &S);
 // CSR row pointers of a sorted matrix (n_rows+1 entries).
 void build_row_ptr(const sddmm_coo &S, std::vector<int32_t> &row_ptr);

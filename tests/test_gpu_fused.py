@@ -1,0 +1,145 @@
+"""The forms around the SDDMM on the GPU, through the C ABI: row-wise softmax of the sampled
+products (on its own and as sddmm_execute_softmax) and the CSR SpMM that consumes them, against the
+CPU oracle.  Softmax: relative 1e-5 per entry (terms are positive: no cancellation).  SpMM:
+1e-5*sqrt(row length) relative to sum|x*h| (signed terms)."""
+import numpy as np
+import pytest
+import torch
+
+from sddmm_gpu_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def softmax_ok(got, want):
+    assert got.shape == want.shape and np.all(np.isfinite(got))
+    bad = np.abs(got.astype(np.float64) - want) > 1e-5 * np.abs(want) + 1e-37
+    assert not bad.any(), (int(bad.sum()), float(np.abs(got - want).max()))
+
+
+@pytest.mark.parametrize("cfg,scale", [(1, 1.0), (2, 1.0), (3, 0.05), (5, 2.0 ** -6)])
+def test_row_softmax_matches_oracle(oracle, cfg, scale):
+    d = synth.make(cfg, scale)
+    dev = torch.device(DEV)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(d["nnz"], generator=g) * 4.0
+    rp = d["row_ptr"].to(dev); xd = x.to(dev); out = torch.full_like(xd, float("nan"))
+    capi.row_softmax(d["n_rows"], rp.data_ptr(), xd.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    want = oracle.row_softmax(d["row_ptr"].numpy(), x.numpy())
+    softmax_ok(out.cpu().numpy(), want)
+    # in place, and the closed form: equal logits -> 1 / row length
+    capi.row_softmax(d["n_rows"], rp.data_ptr(), xd.data_ptr(), xd.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(xd, out)
+    ones = torch.full((d["nnz"],), 3.25, device=dev)
+    capi.row_softmax(d["n_rows"], rp.data_ptr(), ones.data_ptr(), ones.data_ptr())
+    deg = np.diff(d["row_ptr"].numpy())
+    assert np.allclose(ones.cpu().numpy(), 1.0 / deg[d["row_ind"].numpy()], rtol=1e-6, atol=0)
+
+
+def test_row_softmax_edge_rows(oracle):
+    # empty rows, rows of 1, 64, 65, 512, 513 and 5000 entries (the register path ends at 512)
+    lens = [0, 1, 0, 64, 65, 512, 513, 5000, 0, 2, 511]
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    rng = np.random.default_rng(1)
+    x = rng.normal(0, 10, rp[-1]).astype(np.float32)
+    x[rp[5]] = 80.0; x[rp[7] + 17] = -90.0
+    dev = torch.device(DEV)
+    xd = torch.from_numpy(x).to(dev); out = torch.full_like(xd, float("nan"))
+    capi.row_softmax(len(lens), torch.from_numpy(rp).to(dev).data_ptr(), xd.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
+    capi.row_softmax(0, 0, 0, 0)  # nothing to do
+
+
+@pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])
+def test_execute_softmax_matches_oracle(oracle, monkeypatch, kernel, K):
+    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+    kid = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}[kernel]
+    d = synth.make(3, 0.03, K=K, seed=12)
+    d["W"] = d["W"] * 8.0; d["H"] = d["H"] * 8.0  # logits of order one
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev)
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    cpu_logits = oracle.sddmm_csr(d["row_ptr"].numpy(), d["col_ind"].numpy(), d["val"].numpy(), d["W"].numpy(), d["H"].numpy())
+    want = oracle.row_softmax(d["row_ptr"].numpy(), cpu_logits)
+    # host-created plan (values inside) and device-created plan (values at execute)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    plan = S.plan(K, 0, 0, kid)
+    plan.execute_softmax(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    # the logits differ from the oracle's by the SDDMM tolerance; a softmax entry moves by at most that (absolute, in the logit)
+    tol = 1e-5 * np.sqrt(K) * np.abs(cpu_logits).max() * 4 + 1e-5
+    assert np.all(np.isfinite(got)) and np.all(np.abs(got - want) <= tol * want + 1e-37)
+    sums = np.bincount(d["row_ind"].numpy(), weights=got.astype(np.float64), minlength=d["n_rows"])
+    assert np.allclose(sums[np.diff(d["row_ptr"].numpy()) > 0], 1.0, atol=1e-5)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev); dv = d["val"].to(dev)
+    p2 = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, 0, 0, kid)
+    out2 = torch.full_like(out, float("nan"))
+    p2.execute_softmax(dv.data_ptr(), W.data_ptr(), H.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    # the two-call form gives the same bits
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out2.data_ptr())
+    capi.row_softmax(d["n_rows"], rp.data_ptr(), out2.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("cfg,scale,K", [(1, 1.0, 32), (2, 1.0, 256), (3, 0.05, 128), (3, 0.02, 100), (3, 0.02, 7), (3, 0.02, 36),
+                                         (5, 2.0 ** -6, 512), (3, 0.01, 2048), (3, 0.01, 2052)])
+def test_spmm_matches_oracle(oracle, cfg, scale, K):
+    d = synth.make(cfg, scale, K=K)
+    dev = torch.device(DEV)
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(d["nnz"], generator=g)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev); xd = x.to(dev); H = d["H"].to(dev).contiguous()
+    Y = torch.full((d["n_rows"], K), float("nan"), device=dev)
+    capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), xd.data_ptr(), K, H.data_ptr(), Y.data_ptr())
+    torch.cuda.synchronize()
+    want, absy = oracle.spmm_csr(d["row_ptr"].numpy(), d["col_ind"].numpy(), x.numpy(), d["H"].numpy(), with_abs=True)
+    got = Y.cpu().numpy()
+    assert np.all(np.isfinite(got))
+    deg = np.diff(d["row_ptr"].numpy()).astype(np.float64)
+    bound = 1e-5 * np.sqrt(np.maximum(deg, 1.0))[:, None] * absy + 1e-30
+    bad = np.abs(got.astype(np.float64) - want) > bound
+    assert not bad.any(), (int(bad.sum()), float(np.abs(got - want).max()))
+    assert np.all(got[deg == 0] == 0)
+    # closed form: H of ones -> every output column is the row sum of x
+    ones = torch.ones_like(H)
+    capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), xd.data_ptr(), K, ones.data_ptr(), Y.data_ptr())
+    torch.cuda.synchronize()
+    rs = np.bincount(d["row_ind"].numpy(), weights=x.numpy().astype(np.float64), minlength=d["n_rows"])
+    ab = np.bincount(d["row_ind"].numpy(), weights=np.abs(x.numpy()).astype(np.float64), minlength=d["n_rows"])
+    assert np.all(np.abs(Y.cpu().numpy()[:, K // 2] - rs) <= 1e-5 * np.sqrt(np.maximum(deg, 1.0)) * ab + 1e-30)
+
+
+def test_attention_chain_and_errors(oracle):
+    """softmax(S .* W H^T) H end to end on the bag-of-words shape, and the argument checks."""
+    K = 64
+    d = synth.make(2, 0.5, K=K)
+    d["W"] = d["W"] * 3.0
+    dev = torch.device(DEV)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), np.ones(d["nnz"], np.float32))
+    plan = S.plan(K)
+    W = d["W"].to(dev); H = d["H"].to(dev); rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
+    att = torch.empty(d["nnz"], device=dev); Y = torch.empty(d["n_rows"], K, device=dev)
+    plan.execute_softmax(0, W.data_ptr(), H.data_ptr(), att.data_ptr())
+    capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), att.data_ptr(), K, H.data_ptr(), Y.data_ptr())
+    torch.cuda.synchronize()
+    logits = oracle.sddmm_csr(d["row_ptr"].numpy(), d["col_ind"].numpy(), np.ones(d["nnz"], np.float32), d["W"].numpy(), d["H"].numpy())
+    want = oracle.spmm_csr(d["row_ptr"].numpy(), d["col_ind"].numpy(), oracle.row_softmax(d["row_ptr"].numpy(), logits), d["H"].numpy())
+    # a convex combination of H rows: compare against the scale of H
+    assert np.abs(Y.cpu().numpy() - want).max() <= 1e-4 * np.abs(d["H"].numpy()).max()
+    with pytest.raises(capi.SddmmError) as e:
+        capi.spmm_csr(5, 5, 3, rp.data_ptr(), 0, 0, K, 0, Y.data_ptr())
+    assert e.value.code == capi.ERR_ARG
+    with pytest.raises(capi.SddmmError) as e:
+        capi.spmm_csr(5, 5, 3, rp.data_ptr(), ci.data_ptr(), att.data_ptr(), 0, H.data_ptr(), Y.data_ptr())
+    assert e.value.code == capi.ERR_ARG
+    with pytest.raises(capi.SddmmError) as e:
+        capi.row_softmax(5, 0, att.data_ptr(), att.data_ptr())
+    assert e.value.code == capi.ERR_ARG

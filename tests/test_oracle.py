@@ -224,3 +224,71 @@ def test_restatements_match_reference_header(oracle, seed):
         if nb and not (j >= 1 and nb == 1):
             assert np.array_equal(mine["last_idx_block"][j][lo:nb], ref["last_idx_block"][j][lo:nb]), j
     assert np.array_equal(oracle.initial(n, 7), oracle.ref_initial(n, 7))
+
+
+# ------------------------------------------------- row softmax and SpMM ---
+
+def test_row_softmax_closed_forms(oracle):
+    rng = np.random.default_rng(3)
+    rows, cols = rand_sorted_coo(rng, 60, 80, 900)
+    rp = row_ptr_of(rows, 60)
+    deg = np.diff(rp)
+    # equal logits -> 1 / row length, whatever the common value
+    for c in (0.0, -7.5, 88.0):
+        out = oracle.row_softmax(rp, np.full(len(rows), c, np.float32))
+        assert np.allclose(out, 1.0 / deg[rows], rtol=1e-7, atol=0)
+    x = rng.normal(0, 3, len(rows)).astype(np.float32)
+    out = oracle.row_softmax(rp, x)
+    sums = np.bincount(rows, weights=out.astype(np.float64), minlength=60)
+    assert np.allclose(sums[deg > 0], 1.0, atol=1e-6) and np.all(sums[deg == 0] == 0)
+    # shift invariance per row (a dropped max or a wrong sign in the exponent fails here) and order preservation
+    shift = rng.integers(-20, 20, 60).astype(np.float32)
+    assert np.allclose(oracle.row_softmax(rp, x + shift[rows]), out, rtol=2e-6, atol=1e-12)
+    r = int(np.argmax(deg)); seg = slice(rp[r], rp[r + 1])
+    assert np.array_equal(np.argsort(x[seg], kind="stable"), np.argsort(out[seg], kind="stable"))
+    # one dominant logit -> 1 for it, 0 for the rest; two entries -> the logistic function
+    x2 = x.copy(); x2[rp[r]] = 1e4
+    o2 = oracle.row_softmax(rp, x2)
+    assert o2[rp[r]] == 1.0 and np.all(o2[rp[r] + 1:rp[r + 1]] == 0)
+    two = oracle.row_softmax(np.array([0, 2], np.int32), np.array([0.3, -1.1], np.float32))
+    assert np.allclose(two, [1 / (1 + np.exp(-1.4)), 1 / (1 + np.exp(1.4))], rtol=1e-6)
+
+
+def test_row_softmax_matches_fp64_brute_force(oracle):
+    rng = np.random.default_rng(4)
+    rows, cols = rand_sorted_coo(rng, 25, 3000, 20000)
+    rp = row_ptr_of(rows, 25)
+    x = rng.normal(0, 5, len(rows)).astype(np.float32)
+    out = oracle.row_softmax(rp, x)
+    for r in range(25):
+        seg = x[rp[r]:rp[r + 1]].astype(np.float64)
+        if len(seg):
+            e = np.exp(seg - seg.max())
+            assert np.allclose(out[rp[r]:rp[r + 1]], e / e.sum(), rtol=3e-7, atol=1e-37)
+
+
+def test_spmm_matches_scipy_closed_forms_and_fp64(oracle):
+    rng = np.random.default_rng(5)
+    n, m = 70, 90
+    rows, cols = rand_sorted_coo(rng, n, m, 1500)
+    rp = row_ptr_of(rows, n)
+    x = rng.normal(0, 1, len(rows)).astype(np.float32)
+    for K in (1, 5, 32, 100):
+        H = rng.normal(0, 1, (m, K)).astype(np.float32)
+        Y, absy = oracle.spmm_csr(rp, cols, x, H, with_abs=True)
+        A = sp.csr_matrix((x.astype(np.float64), cols, rp), shape=(n, m))
+        ref = A @ H.astype(np.float64)
+        assert np.all(np.abs(Y - ref) <= 1e-6 * np.sqrt(32) * absy + 1e-30)
+        assert np.allclose(absy, abs(A) @ np.abs(H.astype(np.float64)))
+        assert np.all(Y[np.diff(rp) == 0] == 0)  # rows without entries
+    # one-hot H picks, per row, the sum of the entries whose column maps to that output column
+    K = 8
+    j = rng.integers(0, K, m)
+    H = np.zeros((m, K), np.float32); H[np.arange(m), j] = 1.0
+    xi = rng.integers(1, 6, len(rows)).astype(np.float32)  # small integers: every sum is exact
+    Y = oracle.spmm_csr(rp, cols, xi, H)
+    want = np.zeros((n, K)); np.add.at(want, (rows, j[cols]), xi)
+    assert np.array_equal(Y, want.astype(np.float32))
+    # all ones: the row sums, exactly
+    Y = oracle.spmm_csr(rp, cols, xi, np.ones((m, 3), np.float32))
+    assert np.array_equal(Y[:, 1], np.bincount(rows, weights=xi, minlength=n).astype(np.float32))
