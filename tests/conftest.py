@@ -13,7 +13,30 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
-def parity_report(gpu, cpu, K, absdot=None, cond_limit=100.0):
+PARITY_LOG = []  # (label, report) of every full comparison of this session, written out at its end
+
+
+def record_parity(label, rep):
+    PARITY_LOG.append((label, rep))
+
+
+def pytest_sessionfinish(session, exitstatus):
+    # the per-case figures (strict count, worst relative and norm-wise error, the oracle's own
+    # strict count against fp64) as one JSON line per case, where a run's output is collected
+    if not PARITY_LOG:
+        return
+    import json
+    out = os.path.join(ROOT, "gpurun_out")
+    try:
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "parity_report.jsonl"), "w") as f:
+            for label, rep in PARITY_LOG:
+                f.write(json.dumps(dict(case=label, **rep)) + "\n")
+    except OSError:
+        pass
+
+
+def parity_report(gpu, cpu, K, absdot=None, cond_limit=100.0, f64=None):
     """Compares GPU results with the CPU oracle's.
 
     The bar is |gpu - cpu| <= 1e-5*sqrt(K)*|cpu| per nonzero.  A dot product of
@@ -39,6 +62,12 @@ def parity_report(gpu, cpu, K, absdot=None, cond_limit=100.0):
         rep["max_normwise"] = float((diff[pos] / absdot[pos]).max()) if pos.any() else 0.0
     else:
         rep["violations"] = rep["strict_violations"]
+    if f64 is not None:
+        # what fp32 summation order alone costs on this input: how many of the sequential CPU sums, and
+        # how many of the GPU's, miss the strict bound against the fp64 value
+        f64 = np.asarray(f64, np.float64)
+        rep["cpu_vs_f64_strict"] = int((np.abs(cpu - f64) > tol * np.abs(f64)).sum())
+        rep["gpu_vs_f64_strict"] = int((np.abs(gpu - f64) > tol * np.abs(f64)).sum())
     return rep
 
 

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import parity_report
+from conftest import parity_report, record_parity
 from sddmm_gpu_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
@@ -29,7 +29,7 @@ def run(d, kernel, W=None, plan_values=False):
     return out, info
 
 
-@pytest.mark.parametrize("cfg,K", [(3, 128), (3, 256), (4, 64), (5, 512)])
+@pytest.mark.parametrize("cfg,K", [(3, 128), (3, 256), (3, 32), (3, 512), (4, 64), (5, 512), (5, 1024)])
 def test_full_size(oracle, cfg, K):
     dev = torch.device("cuda:0")
     d = synth.make(cfg, 1.0, device=dev, K=K)
@@ -51,9 +51,11 @@ def test_full_size(oracle, cfg, K):
     rows = d["row_ind"][idx].cpu().numpy(); cols = d["col_ind"][idx].cpu().numpy(); vals = d["val"][idx].cpu().numpy()
     W = d["W"].cpu().numpy(); H = d["H"].cpu().numpy()
     cpu = oracle.sddmm_coo(rows, cols, vals, W, H)
-    _, absp = oracle.sddmm_f64(rows, cols, vals, W, H)
-    rep = parity_report(out[idx].cpu().numpy(), cpu, K, absp)
+    f64, absp = oracle.sddmm_f64(rows, cols, vals, W, H)
+    rep = parity_report(out[idx].cpu().numpy(), cpu, K, absp, f64=f64)
+    record_parity(f"full size config {cfg} K={K} nnz={nnz} (sample of 400000)", rep)
     assert rep["violations"] == 0, rep
+    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"] + max(3, rep["cpu_vs_f64_strict"] // 4), rep
     del W, H
 
     # (1b) values kept by the plan in stream order: the same arithmetic, so the same bits

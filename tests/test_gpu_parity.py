@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import parity_report
+from conftest import parity_report, record_parity
 from sddmm_gpu_amd import capi, synth
 
 pytestmark = pytest.mark.gpu
@@ -31,7 +31,12 @@ def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_val
     return out.cpu().numpy(), plan.info()
 
 
-def check(d, out, oracle, K=None):
+def check(d, out, oracle, K=None, label=None):
+    """The bar of every comparison here.  Per nonzero: |gpu - cpu| <= 1e-5*sqrt(K)*|cpu|, or, where the
+    terms of the dot product cancel (condition number above 100), the same tolerance against
+    sum|w h|/100 -- no fp32 summation order meets a relative bound there, the sequential CPU sum
+    included.  So that the relaxed form is not the only gate, the GPU's strict misses against the
+    fp64 value must not outnumber the CPU oracle's own (both counts are in the report)."""
     K = K or d["K"]
     rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
     W = d["W"].numpy(); H = d["H"].numpy()
@@ -39,11 +44,13 @@ def check(d, out, oracle, K=None):
     assert np.array_equal(cpu, oracle.sddmm_coo(rows, cols, vals, W, H))
     f64, absp = oracle.sddmm_f64(rows, cols, vals, W, H)
     assert out.shape == cpu.shape and np.all(np.isfinite(out))
-    rep = parity_report(out, cpu, K, absp)
+    rep = parity_report(out, cpu, K, absp, f64=f64)
+    record_parity(label or f"{d.get('name', 'matrix')} {d['n_rows']}x{d['n_cols']} nnz={d['nnz']} K={K}", rep)
     assert rep["violations"] == 0, rep
+    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"] + max(3, rep["cpu_vs_f64_strict"] // 4), rep
     # the GPU's tree-shaped sum must not be less accurate than the sequential CPU sum
     err_gpu = np.abs(out - f64).max(); err_cpu = np.abs(cpu - f64).max()
-    assert err_gpu <= 2 * err_cpu + 1e-30, (err_gpu, err_cpu)
+    assert err_gpu <= 2 * err_cpu + 1e-30, (err_gpu, err_cpu, rep)
     return rep
 
 
