@@ -229,6 +229,8 @@ typedef struct sddmm_plan_options {
     int32_t dense_permille;     /* least fill of a dense block, in 1/1000           [SDDMM_DENSE_PERMILLE] */
     int32_t dense_rb_group;     /* row blocks swept together by one die             [SDDMM_DENSE_RB_GROUP] */
     int32_t ignore_env;         /* 1: the environment is not consulted                                      */
+    int64_t gather_slab_cols;   /* padded gather streams S in slabs of this many columns [SDDMM_GATHER_SLAB_COLS] */
+    int64_t gather_panel_rows;  /* ... and, inside, in panels of this many listed rows   [SDDMM_GATHER_PANEL_ROWS] */
     int64_t dense_min_nnz;      /* fewer dense nonzeros than this: no dense launch  [SDDMM_DENSE_MIN_NNZ] */
     int64_t panel_bytes;        /* W bytes per row panel of an LDS_TILE stream      [SDDMM_PANEL_BYTES]   */
     int64_t short_row_max;      /* rows with fewer nonzeros go to the short class   [SDDMM_SHORT_ROW_MAX] */

@@ -195,7 +195,7 @@ void default_options(sddmm_plan_options &o)
     o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.gather_lanes = -1; o.gather_padded = -1;
     o.gather_sink = -1; o.row_padded = -1; o.unpadded_tile = -1; o.dense_blocks = -1; o.dense_permille = -1;
     o.dense_rb_group = -1; o.ignore_env = 0;
-    o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
+    o.gather_slab_cols = -1; o.gather_panel_rows = -1; o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
 }
 
 // The environment as an override layer over the caller's options.
@@ -211,7 +211,7 @@ void apply_env_overrides(sddmm_plan_options &o)
     i32("SDDMM_GATHER_G", o.gather_lanes); i32("SDDMM_GATHER_PADDED", o.gather_padded); i32("SDDMM_GATHER_SINK", o.gather_sink);
     i32("SDDMM_ROW_PADDED", o.row_padded); i32("SDDMM_UNPADDED_TILE", o.unpadded_tile); i32("SDDMM_DENSE", o.dense_blocks);
     i32("SDDMM_DENSE_PERMILLE", o.dense_permille); i32("SDDMM_DENSE_RB_GROUP", o.dense_rb_group);
-    i64("SDDMM_DENSE_MIN_NNZ", o.dense_min_nnz); i64("SDDMM_PANEL_BYTES", o.panel_bytes);
+    i64("SDDMM_GATHER_SLAB_COLS", o.gather_slab_cols); i64("SDDMM_GATHER_PANEL_ROWS", o.gather_panel_rows); i64("SDDMM_DENSE_MIN_NNZ", o.dense_min_nnz); i64("SDDMM_PANEL_BYTES", o.panel_bytes);
     i64("SDDMM_SHORT_ROW_MAX", o.short_row_max); i64("SDDMM_STAGE_FACTOR", o.stage_factor);
     i64("SDDMM_SPLIT_MIN_NNZ", o.split_min_nnz);
 }
@@ -476,7 +476,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // H rows read from global memory instead of an LDS tile
     Launch L;
     L.kind = gather ? SDDMM_KERNEL_ROW_GATHER : SDDMM_KERNEL_LDS_TILE;
-    if (gather) { x = (int32_t)std::max<int64_t>(c.n_cols, 1); panel_rows = INT32_MAX; }
+    // (gather form over column slabs: the stream lists S slab by slab, so that the H rows one pass
+    // gathers come from a range small enough to stay in the last-level cache)
+    if (gather) {
+        x = (int32_t)std::max<int64_t>(c.n_cols, 1);
+        if (c.opt.gather_slab_cols > 0) x = (int32_t)std::min<int64_t>(x, c.opt.gather_slab_cols);
+        panel_rows = c.opt.gather_panel_rows > 0 ? (int32_t)std::min<int64_t>(c.opt.gather_panel_rows, INT32_MAX) : INT32_MAX;
+    }
     L.rows = (int64_t)rows.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
     // 12 waves per workgroup measured 2-5 % faster than 16 on slices of 64 and 128, slower on 32
@@ -1212,10 +1218,23 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (!rs.empty()) {
             // short rows: the padded, pipelined kernel reading H from global memory when the
             // rows are short enough for padding to stay cheap; the plain row gather otherwise
-            const int gg = opt.gather_lanes > 0 ? opt.gather_lanes : 8;
-            const bool padded = opt.gather_padded != 0 && pick_tile_variant(kt, gg).G != 0 && (!rl.empty() || D.n_dense > 0);
-            if (padded) { if (int rc = add_tile(c, rs, 0, 0, gg, kt, nullptr, true)) return rc; }
-            else if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
+            // An H far larger than the caches (every die's 4 MB of L2, 32 MB together) and no tiled class:
+            // every gathered H row would cross the fabric (R-MAT 2^22, K=64: 41.8 GB per step for 4.5 GB of
+            // algorithmic bytes, 8.27 ms).  The padded gather then walks S in column slabs whose H rows
+            // come to 32 MB, with groups of 4 lanes (runs inside a slab are short): 26.3 GB, 4.96 ms.
+            // Narrower slabs lose to the W rows re-read per (row, slab) run, wider ones to H misses.
+            const bool huge_h = rl.empty() && D.n_dense == 0 && (int64_t)n_cols * K * 4 > ((int64_t)256 << 20);
+            int gg = opt.gather_lanes > 0 ? opt.gather_lanes : 8;
+            if (huge_h && opt.gather_lanes <= 0 && opt.gather_slab_cols != 0 && pick_tile_variant(kt, 4).G) gg = 4;
+            const bool slabs = huge_h && opt.gather_slab_cols != 0 && opt.gather_padded != 0 && pick_tile_variant(kt, gg).G != 0;
+            const bool padded = opt.gather_padded != 0 && pick_tile_variant(kt, gg).G != 0 && (!rl.empty() || D.n_dense > 0 || slabs);
+            if (padded) {
+                const int64_t keep = c.opt.gather_slab_cols;
+                if (slabs && keep < 0) c.opt.gather_slab_cols = std::max<int64_t>(1024, ((int64_t)32 << 20) / ((int64_t)K * 4));
+                const int rc = add_tile(c, rs, 0, 0, gg, kt, nullptr, true);
+                c.opt.gather_slab_cols = keep;
+                if (rc) return rc;
+            } else if (int rc = add_row_gather(c, rs, rs.size() == ne.size())) return rc;
         }
         I.kernel = (P->launches.size() == 1 && !P->launches[0].dfn) ? P->launches[0].kind : SDDMM_KERNEL_HYBRID;
         I.class_nnz[0] = nl; I.class_nnz[1] = 0; I.class_nnz[2] = nsh;

@@ -120,3 +120,31 @@ def test_dense_block_launch(oracle, cfg, scale, K):
         plan.execute_epilogue(src, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
         torch.cuda.synchronize()
         residual_ok(out.cpu().numpy(), d, oracle, K)
+
+
+@pytest.mark.parametrize("K,slab,panel", [(64, 4096, -1), (64, 1000, 3000), (128, 2048, -1), (256, 512, -1), (32, 8192, 100)])
+def test_padded_gather_over_column_slabs(oracle, K, slab, panel):
+    """The padded gather walking S slab by slab (and row panel by row panel), the form AUTO builds when H is far
+    larger than the caches: same results as the oracle, values in every mode."""
+    d = synth.make(4, 2.0 ** -7, K=K)
+    dev = torch.device(DEV)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev); dv = d["val"].to(dev)
+    opts = capi.PlanOptions.defaults(kernel=capi.KERNEL_ROW_GATHER, row_padded=1, gather_lanes=4 if K <= 128 else 8,
+                                     gather_slab_cols=slab, gather_panel_rows=panel, ignore_env=1)
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, keep=(rp, ci), options=opts)
+    info = plan.info()
+    assert info["padded_positions"] >= d["nnz"]
+    W = d["W"].to(dev); H = d["H"].to(dev)
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(dv.data_ptr(), W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    check(d, out.cpu().numpy(), oracle, K)
+    plan.set_values(dv.data_ptr())
+    out2 = torch.full_like(out, float("nan"))
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    out2.fill_(float("nan"))
+    plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out2.data_ptr(), capi.EPILOGUE_RESIDUAL)
+    torch.cuda.synchronize()
+    residual_ok(out2.cpu().numpy(), d, oracle, K)
