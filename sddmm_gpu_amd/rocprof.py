@@ -152,6 +152,7 @@ def as_text(s):
     lines = [f"rocprofv3 summary of {s['profile_dir']} (passes: {', '.join(s['passes'])}), made by python3 -m sddmm_gpu_amd.rocprof {s['profile_dir']}",
              "each pass is a run of its own on the MI355X box, from the repository root, after cd /tmp && export TMPDIR=/tmp && cd back:"]
     lines += ["  " + c for c in s["commands"]]
+    lines.append("(the line each run prints is kept as run.json in its pass directory: it carries the number of steps the run issued)")
     lines.append("(bytes per step = counter in KiB x 1024 x scale factor, summed over the kernels of one sddmm_execute; the scale factor is")
     lines.append(" the known size of the copy probe of the same run divided by what the counter reads for it)")
     for cname, h in s.get("hbm", {}).items():
