@@ -189,6 +189,7 @@ int64_t env_i64(const char *name, int64_t dflt)
 
 void default_options(sddmm_plan_options &o)
 {
+    memset(&o, 0, sizeof o);
     o.kernel = SDDMM_KERNEL_AUTO;
     o.tile_size_x = 0; o.tile_size_y = 0;
     o.k_slice = -1; o.tile_lanes = -1; o.tile_waves = -1; o.tile_assign = -1; o.tile_few_blocks = -1;
@@ -1545,11 +1546,17 @@ bool decode_pointer(const sddmm_plan *P, uint64_t code, void **p)
 
 bool same_options(const sddmm_plan_options &a, const sddmm_plan_options &b)
 {
-    sddmm_plan_options x = a, y = b;
-    x.ignore_env = y.ignore_env = 0;  // how the values got there is not part of the key
-    if (x.tile_lanes < 0) x.tile_lanes = 0;
-    if (y.tile_lanes < 0) y.tile_lanes = 0;
-    return memcmp(&x, &y, sizeof x) == 0;
+    // field by field (the structure may hold padding); how the values got there (ignore_env) is not part of the key
+    const int la = a.tile_lanes < 0 ? 0 : a.tile_lanes, lb = b.tile_lanes < 0 ? 0 : b.tile_lanes;
+    return a.kernel == b.kernel && a.tile_size_x == b.tile_size_x && a.tile_size_y == b.tile_size_y && a.k_slice == b.k_slice &&
+           la == lb && a.tile_waves == b.tile_waves && a.tile_assign == b.tile_assign && a.tile_few_blocks == b.tile_few_blocks &&
+           a.tile_short_batches == b.tile_short_batches && a.tile_deal == b.tile_deal && a.tile_runs == b.tile_runs &&
+           a.gather_lanes == b.gather_lanes && a.gather_padded == b.gather_padded && a.gather_sink == b.gather_sink &&
+           a.row_padded == b.row_padded && a.unpadded_tile == b.unpadded_tile && a.dense_blocks == b.dense_blocks &&
+           a.dense_permille == b.dense_permille && a.dense_rb_group == b.dense_rb_group &&
+           a.gather_slab_cols == b.gather_slab_cols && a.gather_panel_rows == b.gather_panel_rows &&
+           a.dense_min_nnz == b.dense_min_nnz && a.panel_bytes == b.panel_bytes && a.short_row_max == b.short_row_max &&
+           a.stage_factor == b.stage_factor && a.split_min_nnz == b.split_min_nnz;
 }
 
 struct FileCloser { FILE *f; ~FileCloser() { if (f) fclose(f); } };
