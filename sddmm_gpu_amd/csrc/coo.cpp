@@ -66,14 +66,19 @@ void parallel_ranges(int64_t n, int64_t grain, const std::function<void(int64_t,
     th.reserve(nt);
     for (int t = 0; t < nt; ++t) {
         int64_t b = n * t / nt, e = n * (t + 1) / nt;
-        th.emplace_back([&f, &err, &err_mu, b, e, t] {
+        auto body = [&f, &err, &err_mu, b, e, t] {
             try {
                 f(b, e, t);
             } catch (...) {
                 std::lock_guard<std::mutex> g(err_mu);
                 if (!err) err = std::current_exception();
             }
-        });
+        };
+        try {
+            th.emplace_back(body);
+        } catch (...) {
+            body();  // no thread to be had: this range runs here
+        }
     }
     for (auto &x : th) x.join();
     if (err) std::rethrow_exception(err);
@@ -92,8 +97,8 @@ void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t
     std::mutex err_mu;
     std::vector<std::thread> th;
     th.reserve(nt);
-    for (int t = 0; t < nt; ++t)
-        th.emplace_back([&, t] {
+    for (int t = 0; t < nt; ++t) {
+        auto body = [&, t] {
             try {
                 for (;;) {
                     const int64_t b = next.fetch_add(chunk);
@@ -105,7 +110,13 @@ void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t
                 std::lock_guard<std::mutex> g(err_mu);
                 if (!err) err = std::current_exception();
             }
-        });
+        };
+        try {
+            th.emplace_back(body);
+        } catch (...) {
+            body();  // no thread to be had: the chunks left are taken here
+        }
+    }
     for (auto &x : th) x.join();
     if (err) std::rethrow_exception(err);
 }
@@ -344,7 +355,13 @@ int sddmm_cpu(const sddmm_coo *S, int32_t K, const float *W, const float *H, flo
         };
         std::vector<std::thread> th;
         th.reserve((size_t)nt);
-        for (int t = 1; t < nt; ++t) th.emplace_back(work);
+        for (int t = 1; t < nt; ++t) {
+            try {
+                th.emplace_back(work);
+            } catch (...) {
+                break;  // fewer threads: the shared counter hands the chunks to those that run
+            }
+        }
         work();
         for (auto &x : th) x.join();
     } catch (const std::exception &e) {

@@ -131,7 +131,7 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
     try {
         S->n_rows = n_rows; S->n_cols = n_cols; S->nnz = nnz;
         S->rows.resize((size_t)nnz); S->cols.resize((size_t)nnz); S->vals.resize((size_t)nnz);
-    } catch (const std::bad_alloc &) {
+    } catch (const std::exception &) {
         delete S;
         return fail(SDDMM_ERR_NOMEM, "sddmm_read_mtx: out of memory for %lld nonzeros", (long long)nnz);
     }
@@ -149,19 +149,25 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
     }
     for (int t = 1; t <= nt; ++t) if (cb[t] < cb[t - 1]) cb[t] = cb[t - 1];
     std::vector<int64_t> cnt((size_t)nt + 1, 0);
-    {
-        std::vector<std::thread> th;
-        for (int t = 0; t < nt; ++t)
-            th.emplace_back([&, t] {
-                int64_t c = 0;
-                for (const char *q = cb[t]; q < cb[t + 1];) {
-                    const char *le = line_end(q, cb[t + 1]);
-                    if (!blank_or_comment(q, le)) ++c;
-                    q = le + 1;
-                }
-                cnt[t + 1] = c;
-            });
-        for (auto &x : th) x.join();
+    auto over_chunks = [&](const std::function<void(int)> &f) {  // f(chunk) on one thread per chunk
+        try {
+            parallel_ranges(nt, 1, [&](int64_t b, int64_t e2, int) { for (int64_t t = b; t < e2; ++t) f((int)t); });
+            return true;
+        } catch (const std::exception &) {
+            return false;
+        }
+    };
+    if (!over_chunks([&](int t) {
+            int64_t c = 0;
+            for (const char *q = cb[t]; q < cb[t + 1];) {
+                const char *le = line_end(q, cb[t + 1]);
+                if (!blank_or_comment(q, le)) ++c;
+                q = le + 1;
+            }
+            cnt[t + 1] = c;
+        })) {
+        delete S;
+        return fail(SDDMM_ERR_NOMEM, "sddmm_read_mtx: out of memory");
     }
     for (int t = 0; t < nt; ++t) cnt[t + 1] += cnt[t];
     if (cnt[nt] < nnz) {
@@ -171,10 +177,7 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
     }
     std::vector<int> err((size_t)nt, 0);
     std::vector<int64_t> err_line((size_t)nt, 0);
-    {
-        std::vector<std::thread> th;
-        for (int t = 0; t < nt; ++t)
-            th.emplace_back([&, t] {
+    if (!over_chunks([&](int t) {
                 int64_t i = cnt[t];
                 for (const char *q = cb[t]; q < cb[t + 1] && i < nnz;) {
                     const char *le = line_end(q, cb[t + 1]);
@@ -192,8 +195,9 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
                     }
                     q = le + 1;
                 }
-            });
-        for (auto &x : th) x.join();
+        })) {
+        delete S;
+        return fail(SDDMM_ERR_NOMEM, "sddmm_read_mtx: out of memory");
     }
     for (int t = 0; t < nt; ++t)
         if (err[t]) {
@@ -208,7 +212,7 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
         for (int64_t i = 0; i < nnz; ++i) extra += S->rows[i] != S->cols[i];
         try {
             S->rows.reserve((size_t)(nnz + extra)); S->cols.reserve((size_t)(nnz + extra)); S->vals.reserve((size_t)(nnz + extra));
-        } catch (const std::bad_alloc &) {
+        } catch (const std::exception &) {
             delete S;
             return fail(SDDMM_ERR_NOMEM, "sddmm_read_mtx: out of memory");
         }
@@ -218,7 +222,12 @@ extern "C" int sddmm_read_mtx(const char *path, sddmm_coo **out)
             }
         S->nnz = nnz + extra;
     }
-    S->sorted = check_sorted(*S) ? 1 : 0;
+    try {
+        S->sorted = check_sorted(*S) ? 1 : 0;
+    } catch (const std::exception &) {
+        delete S;
+        return fail(SDDMM_ERR_NOMEM, "out of memory while checking the order of '%s'", path);
+    }
     *out = S;
     return SDDMM_OK;
 }
@@ -270,7 +279,7 @@ extern "C" int sddmm_read_bin(const char *path, sddmm_coo **out)
     size_t n = (size_t)h.nnz;
     try {
         S->rows.resize(n); S->cols.resize(n); S->vals.resize(n);
-    } catch (const std::bad_alloc &) {
+    } catch (const std::exception &) {
         delete S; fclose(f);
         return fail(SDDMM_ERR_NOMEM, "sddmm_read_bin: out of memory");
     }
@@ -284,7 +293,12 @@ extern "C" int sddmm_read_bin(const char *path, sddmm_coo **out)
             delete S;
             return fail(SDDMM_ERR_RANGE, "sddmm_read_bin: entry %zu of '%s' lies outside the matrix", i, path);
         }
-    S->sorted = check_sorted(*S) ? 1 : 0;
+    try {
+        S->sorted = check_sorted(*S) ? 1 : 0;
+    } catch (const std::exception &) {
+        delete S;
+        return fail(SDDMM_ERR_NOMEM, "out of memory while checking the order of '%s'", path);
+    }
     *out = S;
     return SDDMM_OK;
 }

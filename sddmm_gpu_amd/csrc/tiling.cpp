@@ -94,7 +94,7 @@ int build_tiling(int64_t n_rows, int64_t n_cols, int64_t nnz_all, const int32_t 
         T.tiled_ind.resize((size_t)nnz);
         T.active_row.resize((size_t)acc_s);
         T.active_end.resize((size_t)acc_s);
-    } catch (const std::bad_alloc &) {
+    } catch (const std::exception &) {
         return fail(SDDMM_ERR_NOMEM, "tiling: out of memory (%lld nonzeros, %lld row runs)", (long long)nnz, (long long)acc_s);
     }
     // pass 2: write the permutation and the active-row lists
@@ -161,7 +161,7 @@ extern "C" int sddmm_tiling_create(const sddmm_coo *S, int32_t tile_size_x, int3
         std::vector<int32_t> rp;
         build_row_ptr(*S, rp);
         rc = build_tiling(S->n_rows, S->n_cols, S->nnz, rp.data(), S->cols.data(), tile_size_x, tile_size_y, *T, nullptr, 0);
-    } catch (const std::bad_alloc &) {
+    } catch (const std::exception &) {
         rc = fail(SDDMM_ERR_NOMEM, "sddmm_tiling_create: out of memory");
     }
     if (rc) { delete T; return rc; }
