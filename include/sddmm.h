@@ -41,11 +41,15 @@ enum {
  * (it builds a HYBRID plan, which may consist of a single family). */
 enum {
     SDDMM_KERNEL_AUTO = 0,
-    SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM */
+    SDDMM_KERNEL_ROW_GATHER = 1, /* W row in VGPRs, H rows gathered from L2/HBM (as a plan: the unpadded stream kernel;
+                                    as the short-row launch of a HYBRID plan: the padded, pipelined gather, over
+                                    column slabs when H is far larger than the caches) */
     SDDMM_KERNEL_LDS_TILE = 2,   /* column tiles of H staged in LDS, W row (re)loaded per row run */
     SDDMM_KERNEL_PANEL = 3,      /* row panels of W resident in VGPRs, column tiles of H swept through LDS */
-    SDDMM_KERNEL_HYBRID = 4,     /* the dense core as DENSE_BLOCK launches, the rest split by row length: long rows ->
-                                    LDS_TILE, short rows -> ROW_GATHER (what AUTO builds) */
+    SDDMM_KERNEL_HYBRID = 4,     /* what AUTO builds: (from K = 512 on, or when asked) the dense core as a DENSE_BLOCK
+                                    launch, the rest split by row length: rows with at least 2 nonzeros per column
+                                    tile -> LDS_TILE (padded tile kernel), shorter rows -> ROW_GATHER; a class too
+                                    small to pay for its launch joins the other.  Never a PANEL launch. */
     SDDMM_KERNEL_DENSE_BLOCK = 5 /* blocks of 128 heavy rows x 128 popular columns computed whole on the matrix cores,
                                     their nonzeros picked from the result; never a plan of its own, only a launch of a
                                     HYBRID plan (reported by sddmm_execute_profiled) */
@@ -69,11 +73,12 @@ typedef struct sddmm_plan_info {
     int32_t grid, block;  /* launch shape of the main kernel */
     int64_t n_blocks;     /* (row panel, column tile) work items with at least one nonzero */
     int64_t device_bytes; /* device memory owned by the plan */
-    int64_t class_nnz[3]; /* nonzeros handled by LDS_TILE, PANEL, ROW_GATHER launches */
+    int64_t class_nnz[3]; /* nonzeros handled by LDS_TILE, PANEL (explicit PANEL plans only), ROW_GATHER launches;
+                             with dense_nnz they add up to nnz */
     int64_t class_rows[3];
     int64_t padded_positions; /* stream positions of the LDS_TILE launches, padding included */
     int64_t short_batches;    /* batches of 64 of those positions that run in half the steps */
-    double plan_ms;       /* host time spent in the tiling pass + upload */
+    double plan_ms;       /* host time spent in the tiling pass + upload (a loaded plan: in reading the file) */
     int64_t dense_nnz;    /* nonzeros handled by the DENSE_BLOCK launch */
     int64_t dense_blocks; /* its 128 x 128 blocks */
 } sddmm_plan_info;
