@@ -148,3 +148,62 @@ def test_padded_gather_over_column_slabs(oracle, K, slab, panel):
     plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out2.data_ptr(), capi.EPILOGUE_RESIDUAL)
     torch.cuda.synchronize()
     residual_ok(out2.cpu().numpy(), d, oracle, K)
+
+
+def test_concurrent_executes_on_one_plan_and_concurrent_plan_creation(oracle):
+    """The header's promise: a plan is immutable, sddmm_execute may be called from several threads on the same plan
+    (each on its own stream, outputs apart); plans may also be built concurrently."""
+    import threading
+    K = 128
+    d = synth.make(3, 0.05, K=K, seed=19)
+    dev = torch.device(DEV)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    opts = capi.PlanOptions.defaults(split_min_nnz=0, ignore_env=1)
+    plan = S.plan(K, options=opts)
+    W = d["W"].to(dev); H = d["H"].to(dev)
+    ref = torch.empty(d["nnz"], device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), ref.data_ptr())
+    torch.cuda.synchronize()
+    check(d, ref.cpu().numpy(), oracle, K)
+    n_threads, reps = 4, 8
+    outs = [torch.full((d["nnz"],), float("nan"), device=dev) for _ in range(n_threads)]
+    streams = [torch.cuda.Stream() for _ in range(n_threads)]
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(reps):
+                plan.execute(0, W.data_ptr(), H.data_ptr(), outs[i].data_ptr(), streams[i].cuda_stream)
+            streams[i].synchronize()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    th = [threading.Thread(target=worker, args=(i,)) for i in range(n_threads)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o, ref)
+    # plans built at the same time from the same host matrix are the same plan
+    plans = [None] * 3
+
+    def builder(i):
+        try:
+            plans[i] = S.plan(K, options=opts)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    th = [threading.Thread(target=builder, args=(i,)) for i in range(3)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not errors, errors
+    for p in plans:
+        o = torch.empty(d["nnz"], device=dev)
+        p.execute(0, W.data_ptr(), H.data_ptr(), o.data_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(o, ref)
