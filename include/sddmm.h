@@ -14,7 +14,10 @@
  * error code and never throw; sddmm_last_error() gives the message of the
  * last failure on the calling thread.  "host" / "device" say where a pointer
  * must live.  Plans are immutable after creation: sddmm_execute may be called
- * from several threads on the same plan (each call on its own stream).
+ * from several threads on the same plan (each call on its own stream) -- with
+ * one exception: a plan that works in K slices (sddmm_plan_info.k_slice < K,
+ * i.e. K > 128) keeps the partial results between its slices in a buffer of
+ * its own, so executes of such a plan must not overlap in time.
  */
 #ifndef SDDMM_H
 #define SDDMM_H

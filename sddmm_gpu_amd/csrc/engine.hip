@@ -39,8 +39,8 @@ struct Launch {
     KernelFn fn = nullptr;   // stream kernels
     PanelFn pfn = nullptr;   // panel kernel
     TileFn tfn = nullptr;        // tile kernel (values in stream order, first K slice); null: not a tile launch
-    TileFn tfns[5][2] = {};      // [values in stream order / in sorted order / none / residual epilogue with values
-                                 //  in stream order / in sorted order][first K slice / later slices]
+    TileFn tfns[5][3] = {};      // [values in stream order / in sorted order / none / residual epilogue with values
+                                 //  in stream order / in sorted order][the only K slice / first of several / a later one]
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
@@ -59,7 +59,7 @@ struct Launch {
 struct sddmm_plan {
     sddmm_plan_info info{};
     std::vector<Launch> launches;
-    struct Owned { void *p; size_t bytes; };
+    struct Owned { void *p; size_t bytes; bool scratch = false; };  // scratch: contents need not be kept (plan files)
     std::vector<Owned> owned;   // device allocations freed with the plan (sizes kept for sddmm_plan_save)
     uint64_t pattern_hash = 0;  // of the CSR pattern the plan was built for (see pattern_hash_host)
     const int32_t *d_row_ptr = nullptr, *d_col = nullptr;
@@ -234,8 +234,8 @@ int resolve_functions(Launch &L)
     case 3: {
         const TileVariant tv{L.fn_g, L.fn_kpl};
         for (int vm = 0; vm < 5; ++vm)
-            for (int ac = 0; ac < 2; ++ac) {
-                L.tfns[vm][ac] = tile_kernel(tv, vm, L.fn_gather != 0, ac != 0, L.fn_nwaves);
+            for (int ac = 0; ac < 3; ++ac) {
+                L.tfns[vm][ac] = tile_kernel(tv, vm, L.fn_gather != 0, ac, L.fn_nwaves);
                 if (!L.tfns[vm][ac]) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for lanes %d x %d", tv.G, tv.KPL);
                 HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
             }
@@ -489,7 +489,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     // 12 waves per workgroup measured 2-5 % faster than 16 on slices of 64 and 128, slower on 32
     int nwaves = gather ? 4 : (int)(c.opt.tile_waves > 0 ? c.opt.tile_waves : (ks >= 64 ? 12 : 16));
     if (!gather && nwaves != 12) nwaves = 16;
-    if (!tv.G || !tile_kernel(tv, 0, gather, false, nwaves)) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
+    if (!tv.G || !tile_kernel(tv, 0, gather, 0, nwaves)) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
     L.fn_kind = 3; L.fn_g = tv.G; L.fn_kpl = tv.KPL; L.fn_gather = gather; L.fn_nwaves = nwaves;
     const int G = tv.G;
     L.nnz = list_nnz(c, rows);
@@ -867,6 +867,17 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     a.perm = d_perm; a.scol = d_scol; a.grow = d_grow; a.unit_ptr = d_uptr; a.unit_tile = d_utile;
     L.sval = d_sval; L.perm = d_perm;
     a.n_units = (int32_t)unit_tile.size(); a.tile_x = x; a.n_cols = (int32_t)c.n_cols; a.K = c.K;
+    if (ks < c.K) {
+        // K slices: the partial results stay in stream order between the slices (coalesced stores and loads); only
+        // the last slice writes out.  One fp32 per stream position, owned by the plan: executes of a sliced plan
+        // that overlap in time would share it.
+        float *d_part = nullptr;
+        const size_t bytes = ((size_t)np + kStreamSlack) * 4;
+        HIP_TRY(hipMalloc((void **)&d_part, bytes));
+        c.P->owned.push_back({d_part, bytes, true});
+        c.dev_bytes += (int64_t)bytes;
+        a.part = d_part;
+    }
     if (gather) {
         float *d_sink = nullptr;
         if (int rc = c.up(&d_sink, std::vector<float>(256 * 64, 0.f))) return rc;
@@ -1417,9 +1428,12 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.sval = d_val ? nullptr : L.sval;
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
         const int vm = residual ? (ta.sval ? 3 : 4) : ta.sval ? 0 : (val ? 1 : 2);
+        const bool sliced = L.k_slice < I.K;
         for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
             ta.k_off = k_off;
-            hipLaunchKernelGGL(L.tfns[vm][k_off > 0], dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
+            ta.to_part = sliced && k_off + L.k_slice < I.K;
+            hipLaunchKernelGGL(L.tfns[vm][!sliced ? 0 : k_off == 0 ? 1 : 2], dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds,
+                               stream, ta);
         }
     } else {
         KArgs a = L.ka;
@@ -1506,14 +1520,15 @@ struct PlanFileHeader {
     char build[40];
 };
 constexpr char kPlanMagic[8] = {'S', 'D', 'D', 'M', 'M', 'P', 'L', 'N'};
-constexpr uint32_t kPlanVersion = 2;
+constexpr uint32_t kPlanVersion = 3;
+constexpr uint64_t kScratchBit = 1ull << 63;
 constexpr uint64_t kBorrowedRowPtr = (1ull << 63) | 1, kBorrowedCol = (1ull << 63) | 2;
 
 // every pointer of a launch that refers to memory the plan owns
 void launch_pointer_fields(Launch &L, std::vector<void *> &fields)
 {
     fields = {&L.ka.perm, &L.ka.scol, &L.ka.seg_row, &L.ka.batch_seg, &L.ka.batch_mask, &L.ka.items,
-            &L.ta.perm, &L.ta.scol, &L.ta.grow, &L.ta.scol16, &L.ta.pbase, &L.ta.btype, &L.ta.sink, &L.ta.unit_ptr,
+            &L.ta.perm, &L.ta.scol, &L.ta.grow, &L.ta.scol16, &L.ta.pbase, &L.ta.btype, &L.ta.part, &L.ta.sink, &L.ta.unit_ptr,
             &L.ta.unit_tile, &L.ta.items,
             &L.pa.slot_row, &L.pa.panel_tiles,
             &L.da.slot_rows, &L.da.slot_cols, &L.da.slot_range, &L.da.nz_p, &L.da.nz_rc,
@@ -1610,12 +1625,15 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
     int64_t total = 0;
     {
         uint64_t at = (uint64_t)data_at;
-        for (uint64_t bytes : sizes) {
+        for (uint64_t word : sizes) {
+            const bool scratch = (word & kScratchBit) != 0;
+            const uint64_t bytes = word & ~kScratchBit;
             if (bytes == 0 || bytes > ((uint64_t)1 << 40)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged", path);
             void *d = nullptr;
             HIP_TRY(hipMalloc(&d, bytes));
-            P->owned.push_back({d, (size_t)bytes});
+            P->owned.push_back({d, (size_t)bytes, scratch});
             total += (int64_t)bytes;
+            if (scratch) continue;
             for (uint64_t off = 0; off < bytes; off += kPiece)
                 pieces.push_back({(char *)d + off, at + off, (size_t)std::min<uint64_t>(kPiece, bytes - off)});
             at += bytes;
@@ -1739,12 +1757,13 @@ int sddmm_plan_save(const sddmm_plan *plan, const char *path)
         FileCloser fc{f};
         bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(&plan->info, sizeof plan->info, 1, f) == 1 &&
                   fwrite(&plan->options, sizeof plan->options, 1, f) == 1;
-        std::vector<uint64_t> sizes;
-        for (const auto &o : plan->owned) sizes.push_back((uint64_t)o.bytes);
+        std::vector<uint64_t> sizes;  // (bit 63: scratch, no contents in the file)
+        for (const auto &o : plan->owned) sizes.push_back((uint64_t)o.bytes | (o.scratch ? kScratchBit : 0));
         ok = ok && (sizes.empty() || fwrite(sizes.data(), 8, sizes.size(), f) == sizes.size());
         ok = ok && (ls.empty() || fwrite((const void *)ls.data(), sizeof(Launch), ls.size(), f) == ls.size());
         std::vector<char> buf;
         for (const auto &o : plan->owned) {
+            if (o.scratch) continue;
             constexpr size_t kPiece = (size_t)64 << 20;
             for (size_t off = 0; ok && off < o.bytes; off += kPiece) {
                 const size_t n = std::min(kPiece, o.bytes - off);

@@ -73,6 +73,8 @@ struct TileArgs {
     const float *val;      // values in sorted order or null
     const float *W, *H;
     float *out;
+    float *part;               // partial results in stream order between the K slices of a sliced launch (else null)
+    int32_t to_part;           // sliced launch: this slice stores to part (every slice but the last)
     float *sink;               // gather form: 256 x 64 floats that take the results of flagged padding positions
     const int32_t *unit_ptr;   // [n_units+1] first stream position of each (row panel, column tile) unit
     const int32_t *unit_tile;  // [n_units] the unit's column tile
@@ -96,8 +98,8 @@ constexpr bool tile_variant_shorts(int G, int KPL, bool gather)
 TileVariant pick_tile_variant(int K, int want_g);
 // vmode: 0 = values in stream order (sval), 1 = values in sorted order (val), 2 = no values
 // gather: H rows from global memory, 4 waves per workgroup (otherwise H tiles in LDS, nwaves = 16 or 12 waves)
-// accumulate: out += instead of out = (K slices after the first)
-TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+// slice: 0 the launch covers all of K, 1 first of several K slices, 2 a later one (see the kernel template)
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
 
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);

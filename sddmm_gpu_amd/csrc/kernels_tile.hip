@@ -17,21 +17,21 @@ TileVariant pick_tile_variant(int K, int want_g)
     return best;
 }
 
-TileFn tile_kernel_part0(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
-TileFn tile_kernel_part1(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
-TileFn tile_kernel_part2(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
-TileFn tile_kernel_part3(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
-TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves);
+TileFn tile_kernel_part0(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
+TileFn tile_kernel_part1(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
+TileFn tile_kernel_part2(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
+TileFn tile_kernel_part3(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
+TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
 
 // vmode: see the kernel template (where S.val comes from, which epilogue)
-TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
+TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, int slice, int nwaves)
 {
     switch (vmode) {
-    case 0: return tile_kernel_part0(v, vmode, gather, accumulate, nwaves);
-    case 1: return tile_kernel_part1(v, vmode, gather, accumulate, nwaves);
-    case 2: return tile_kernel_part2(v, vmode, gather, accumulate, nwaves);
-    case 3: return tile_kernel_part3(v, vmode, gather, accumulate, nwaves);
-    case 4: return tile_kernel_part4(v, vmode, gather, accumulate, nwaves);
+    case 0: return tile_kernel_part0(v, vmode, gather, slice, nwaves);
+    case 1: return tile_kernel_part1(v, vmode, gather, slice, nwaves);
+    case 2: return tile_kernel_part2(v, vmode, gather, slice, nwaves);
+    case 3: return tile_kernel_part3(v, vmode, gather, slice, nwaves);
+    case 4: return tile_kernel_part4(v, vmode, gather, slice, nwaves);
     }
     return nullptr;
 }

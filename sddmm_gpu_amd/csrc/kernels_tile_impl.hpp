@@ -158,10 +158,16 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // the index data of batch b+2 and the W row slice of batch b+1 are in flight.
 // GATHER: no LDS tile; scol holds the column and H rows are read from global
 // memory (the stream is then one unit in row order, for rows too short to tile).
-template <int G, int KPL, int VMODE, int NW, bool GATHER, bool ACC>
+// SLICE: 0 = the launch covers all of K (results go to out); 1 = first of several K slices (partial
+// results go to a.part, in stream order: one coalesced store per batch); 2 = a later slice (adds to the
+// partial result read back from a.part, coalesced, and stores to a.part again or, in the last slice,
+// a.to_part == 0, to out).  Only the last slice touches out, with one scattered store per position.
+template <int G, int KPL, int VMODE, int NW, bool GATHER, int SLICE>
 __global__ __launch_bounds__(NW * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
+    constexpr bool ACC = SLICE == 2;
+    constexpr bool PART = SLICE >= 1;
     extern __shared__ float4 lds_tile[];
     constexpr int K4 = G * KPL;
     constexpr bool RESIDUAL = VMODE >= 3;
@@ -274,7 +280,7 @@ void sddmm_tile_kernel(const TileArgs a)
         // Index data of one batch.  The arrays are addressed as (uniform base of the
         // item) + (32-bit byte offset of the lane), the form that needs no per-lane
         // 64-bit arithmetic, and no load sits behind a branch.
-        struct Meta { uint32_t wrow, p; int col; float sv, old; };
+        struct Meta { uint32_t wrow, p, o; int col; float sv, old; };  // o: byte offset of the position's fp32 slot inside the item
         const uint32_t last = (uint32_t)(end - begin - 1);
         const char *perm_b = reinterpret_cast<const char *>(COMPACT ? a.pbase + begin / G : a.perm + begin);
         const char *scol_b = COMPACT ? reinterpret_cast<const char *>(a.scol16 + begin)
@@ -299,6 +305,7 @@ void sddmm_tile_kernel(const TileArgs a)
                 m.col = *reinterpret_cast<const int *>(scol_b + o4);
             }
             m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
+            m.o = o4;
             o4 += 256;
             og += 256 / G;
             return m;
@@ -319,11 +326,13 @@ void sddmm_tile_kernel(const TileArgs a)
                 m.col = *reinterpret_cast<const int *>(scol_b + t4);
             }
             m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + t4) : 1.0f;
+            m.o = t4;
             return m;
         };
         // ACC (K slices after the first): the previous slices' partial result, requested
-        // one batch ahead of its use
-        auto issue_old = [&](Meta &m) { m.old = ACC ? a.out[GATHER ? (m.p & 0x7fffffffu) : m.p] : 0.f; };
+        // one batch ahead of its use, from the position's own slot of a.part
+        char *part_b = reinterpret_cast<char *>(a.part + begin);
+        auto issue_old = [&](Meta &m) { m.old = ACC ? *reinterpret_cast<const float *>(part_b + m.o) : 0.f; };
         // wrow: float4 index of the row's first element in W
         auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
             const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
@@ -334,10 +343,17 @@ void sddmm_tile_kernel(const TileArgs a)
             for (int j = 0; j < KPL; ++j) w[j] = wbase[j % NB][(j - j % NB) * G];
         };
         float pend_v;  // result of the batch before, not yet stored
-        uint32_t pend_p;
+        uint32_t pend_p, pend_o;
+        const bool to_part = PART && a.to_part != 0;  // (uniform)
         // (gather form: a position whose index carries bit 31 is padding that worked on
         // another row's column; its result goes to a scratch line instead of the output)
         auto flush = [&]() {
+            if constexpr (PART) {
+                if (to_part) {  // (a padding position has a slot of its own)
+                    *reinterpret_cast<float *>(part_b + pend_o) = pend_v;
+                    return;
+                }
+            }
             if constexpr (GATHER) {
                 float *dst = (int32_t)pend_p < 0 ? a.sink + (((blockIdx.x & 255) << 6) + lane) : a.out + pend_p;
                 *dst = pend_v;
@@ -392,6 +408,7 @@ void sddmm_tile_kernel(const TileArgs a)
             if constexpr (RESIDUAL) pend_v = ACC ? m.old - acc[0] : v - acc[0];
             else pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
             pend_p = m.p;
+            pend_o = m.o;
         };
 
         // the type bits of 32 consecutive batches, held in scalar registers

@@ -5,15 +5,15 @@
 
 namespace sddmm {
 
-TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, bool accumulate, int nwaves)
+TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, int slice, int nwaves)
 {
-#define SDDMM_PICK_NW(g, kpl, vm, nw)                                                                       \
-    (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, false, true>                    \
-                : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, false, false>)
+#define SDDMM_PICK_SLICE(g, kpl, vm, nw, ga)                                                                 \
+    (slice == 2 ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, ga, 2>                          \
+     : slice == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, ga, 1>                                        \
+                  : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, ga, 0>)
 #define SDDMM_PICK(g, kpl, vm)                                                                              \
-    (gather ? (accumulate ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), 4, true, true>            \
-                          : (TileFn)sddmm_tile_kernel<g, kpl, vm, 4, true, false>)                          \
-            : (nwaves == 12 ? SDDMM_PICK_NW(g, kpl, vm, 12) : SDDMM_PICK_NW(g, kpl, vm, 16)))
+    (gather ? SDDMM_PICK_SLICE(g, kpl, vm, 4, true)                                                         \
+            : (nwaves == 12 ? SDDMM_PICK_SLICE(g, kpl, vm, 12, false) : SDDMM_PICK_SLICE(g, kpl, vm, 16, false)))
 #define SDDMM_CASE(g, kpl)                                                                                  \
     if (v.G == g && v.KPL == kpl)                                                                           \
         return SDDMM_PICK(g, kpl, 4);
@@ -21,7 +21,7 @@ TileFn tile_kernel_part4(const TileVariant &v, int vmode, bool gather, bool accu
     SDDMM_CASE(16, 4) SDDMM_CASE(16, 8) SDDMM_CASE(32, 4) SDDMM_CASE(32, 8)
 #undef SDDMM_CASE
 #undef SDDMM_PICK
-#undef SDDMM_PICK_NW
+#undef SDDMM_PICK_SLICE
     return nullptr;
 }
 
