@@ -68,7 +68,8 @@ typedef struct sddmm_plan_info {
     int32_t tile_size_x;  /* columns of S (= rows of H) per LDS tile actually used */
     int32_t tile_size_y;  /* row-panel height actually used */
     int32_t k_slice;      /* K elements of each H row resident in LDS at a time (== K: no slicing) */
-    int32_t n_col_tiles, n_row_panels;
+    int32_t n_col_tiles, n_row_panels; /* (n_row_panels: row panels of the stream; with tile_runs = 2 the
+                                          row ranges, one per group of workgroups) */
     int32_t kernel;       /* SDDMM_KERNEL_* actually chosen (HYBRID: more than one launch) */
     int32_t n_launches;   /* kernel launches per sddmm_execute */
     int32_t lanes_per_nnz;
@@ -227,7 +228,10 @@ typedef struct sddmm_plan_options {
     int32_t tile_few_blocks;    /* 0/1 fewest row blocks when staging dominates     [SDDMM_TILE_FEW_BLOCKS] */
     int32_t tile_short_batches; /* 0/1 run ends of <= lanes/2 nonzeros batched apart [SDDMM_TILE_SHORT]    */
     int32_t tile_deal;          /* 0/1 heavy and light tiles dealt to one workgroup [SDDMM_TILE_DEAL]     */
-    int32_t tile_runs;          /* 0/1 runs of neighbouring tiles to one die        [SDDMM_TILE_RUNS]     */
+    int32_t tile_runs;          /* more tiles than workgroups: 0 tiles dealt round-robin,
+                                   1 runs of neighbouring tiles to one die, 2 row ranges
+                                   walked by groups of workgroups of one die (-1:
+                                   2 where rows touch few tiles each, else 1)       [SDDMM_TILE_RUNS]     */
     int32_t gather_lanes;       /* lanes per nonzero of the short-row launch        [SDDMM_GATHER_G]      */
     int32_t gather_padded;      /* 0/1 short rows through the padded gather kernel  [SDDMM_GATHER_PADDED] */
     int32_t gather_sink;        /* 0/1 padding of that stream flagged and dropped   [SDDMM_GATHER_SINK]   */

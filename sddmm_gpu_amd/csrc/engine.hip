@@ -535,6 +535,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         }
         if (grid2d) panel_rows = INT32_MAX;
     }
+    // panel_local (decided below, once the tiling is known): a matrix with more column tiles than
+    // workgroups whose rows touch only a few tiles each (banded shapes) is cut into a few row ranges,
+    // and each range is walked from top to bottom by a group of workgroups of one die that hold the
+    // tiles the rows at the front touch.
+    bool panel_local = false;
+    int pl_slots = 0;      // workgroups per row range
+    int64_t pl_sub = 0;    // batches per piece of an item
     // Short batches (see tile_variant_shorts): the last chunk of a (row, tile) run that holds at
     // most G/2 nonzeros is kept apart from the full chunks, and eight such chunks make a batch of
     // their own, which the kernel runs in half the steps.
@@ -566,20 +573,62 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         n_tiles_all = T.n_tiles;
         const int64_t n_seg = (int64_t)T.active_end.size();
         // row-block boundaries of the 2-D assignment: equal shares of the rows' nonzeros
-        std::vector<int32_t> cut((size_t)shares + 1, INT32_MAX);
-        cut[0] = 0;
-        if (grid2d) {
+        std::vector<int32_t> cut;
+        auto make_cuts = [&](int n_shares) {
+            cut.assign((size_t)n_shares + 1, INT32_MAX);
+            cut[0] = 0;
+            if (!grid2d) return;
             int64_t acc = 0; int sidx = 1;
-            for (size_t i = 0; i < rows.size() && sidx < shares; ++i) {
+            for (size_t i = 0; i < rows.size() && sidx < n_shares; ++i) {
                 acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
-                while (sidx < shares && acc >= L.nnz * sidx / shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
+                while (sidx < n_shares && acc >= L.nnz * sidx / n_shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
             }
-        }
+        };
+        make_cuts(shares);
         auto seg_range = [&](int sh, int32_t j, int64_t *s0, int64_t *s1) {
             const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
             *s0 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh]) - ab);
             *s1 = T.active_ptr[j] + (std::lower_bound(ab, ae, cut[sh + 1]) - ab);
         };
+        // Whole-tile items read a W row once per (row, tile) run, and the workgroups of a die are at
+        // different rows of their tiles, so little of W is found in L2 again: n_seg row slices cross
+        // the L2 boundary.  When a row touches `live` tiles on average and live workgroups fit on a die,
+        // a group of that many workgroups can hold exactly the tiles of the rows it is working on: the
+        // rows are cut into 8 x (groups per die) ranges, one per group; inside a range the tiles go,
+        // in order, to the group's workgroups; a tile's first row in the range is about where the
+        // other workgroups of the group are at that time, so every W row is fetched once per range and
+        // found in L2 by the other tiles that need it.
+        if (grid2d && !xcd_local && shares == 1 && T.n_tiles > c.cus && c.cus % 8 == 0 && !rows.empty() &&
+            (c.opt.tile_runs < 0 || c.opt.tile_runs == 2)) {
+            const int per_die = c.cus / 8;
+            const int live = (int)((n_seg + (int64_t)rows.size() - 1) / (int64_t)rows.size());
+            const int groups = live <= per_die ? per_die / live : 0;
+            if (groups >= 1) {
+                const int want = 8 * groups;
+                make_cuts(want);
+                int64_t n_it = 0, n_ne = 0;
+                for (int32_t j = 0; j < T.n_tiles; ++j) {
+                    const int32_t *ab = T.active_row.data() + T.active_ptr[j], *ae = T.active_row.data() + T.active_ptr[j + 1];
+                    if (ab == ae) continue;
+                    ++n_ne;
+                    // (the tile's rows are ascending: it touches the ranges from its first row's to its last row's)
+                    const int64_t p0 = std::upper_bound(cut.begin(), cut.end() - 1, *ab) - cut.begin() - 1;
+                    const int64_t p1 = std::upper_bound(cut.begin(), cut.end() - 1, *(ae - 1)) - cut.begin() - 1;
+                    n_it += p1 - p0 + 1;
+                }
+                // (every item stages its H tile: the rows' W slices against the tiles staged more than once)
+                if (live >= 2 && (c.opt.tile_runs == 2 || (double)n_seg > 1.5 * ((double)rows.size() + (double)(n_it - n_ne) * x))) {
+                    shares = want;
+                    panel_local = true;
+                    pl_slots = per_die / groups;
+                    // (banded 2^20, K=512, ms per step by batches per wave and piece: 4 -> 4.37, 8 -> 4.25,
+                    // 16 -> 4.24, 32 -> 4.27, 128 -> 4.44; whole tiles in runs of neighbours: 4.56)
+                    pl_sub = (int64_t)nwaves * 16;
+                } else {
+                    make_cuts(shares);
+                }
+            }
+        }
         auto seg_begin = [&](int32_t j, int64_t sg) { return (sg == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[sg - 1]; };
         // Layout with short batches: an item (row block x tile) is a sequence of whole batches.  Its
         // runs are cut into chunks of G positions; a run's last chunk with at most G/2 nonzeros is a
@@ -789,6 +838,35 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
                         const int32_t j = nt >= per_die ? deal[(size_t)die * nt + (size_t)step * per_die + slot] : slot % nt;
                         items.push_back(item_of(sh, j));
                     }
+            } else if (panel_local) {
+                // Range sh belongs to die sh % 8, group sh / 8.  Its items, in tile order, go to the
+                // group's workgroup that is free first (time counted in stream positions).  The waves of
+                // a workgroup split an item into equal contiguous parts, so an item is handed over in
+                // pieces of pl_sub batches: the rows a workgroup touches at one time then lie close
+                // together.  Pieces of one tile follow each other on the same workgroup (staged once).
+                std::vector<std::vector<WorkItem>> seq((size_t)c.cus);
+                for (int sh = 0; sh < shares; ++sh) {
+                    const int die = sh % 8, base = (sh / 8) * pl_slots;
+                    std::vector<int64_t> free_at((size_t)pl_slots, 0);
+                    for (int32_t j : tiles_ne) {
+                        const WorkItem it = item_of(sh, j);
+                        if (it.end <= it.begin) continue;
+                        const int slot = (int)(std::min_element(free_at.begin(), free_at.end()) - free_at.begin());
+                        auto &q = seq[(size_t)((base + slot) * 8 + die)];
+                        const int64_t nb = ((int64_t)it.end - it.begin + 63) / 64;
+                        for (int64_t k0 = 0; k0 < nb; k0 += pl_sub) {
+                            const int64_t k1 = std::min(nb, k0 + pl_sub);
+                            q.push_back({(int32_t)(it.begin + k0 * 64), (int32_t)std::min<int64_t>(it.end, it.begin + k1 * 64),
+                                         (int32_t)(it.batch_base + (shorts ? k0 : 0)), it.tile});
+                        }
+                        free_at[(size_t)slot] += (int64_t)it.end - it.begin;
+                    }
+                }
+                size_t turns = 0;
+                for (auto &q : seq) turns = std::max(turns, q.size());
+                items.assign(turns * (size_t)c.cus, WorkItem{0, 0, 0, 0});
+                for (int b = 0; b < c.cus; ++b)
+                    for (size_t k = 0; k < seq[(size_t)b].size(); ++k) items[k * (size_t)c.cus + (size_t)b] = seq[(size_t)b][k];
             } else if (shares == 1 && c.cus % 8 == 0 && (int64_t)tiles_ne.size() > c.cus &&
                        c.opt.tile_runs != 0) {
                 // More tiles than workgroups (a wide matrix; one item per tile, all rows).  Neighbouring
@@ -870,7 +948,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     if (ks < c.K) {
         // K slices: the partial results stay in stream order between the slices (coalesced stores and loads); only
         // the last slice writes out.  One fp32 per stream position, owned by the plan: executes of a sliced plan
-        // that overlap in time would share it.
+        // that overlap in time would share it.  (Accumulating through out instead, measured on the same build:
+        // banded K=512 5.29 against 4.55 ms; recommender K=256, whose runs of 27 positions make the stores to out
+        // nearly as coalesced, 1.746 against 1.729 ms.)
         float *d_part = nullptr;
         const size_t bytes = ((size_t)np + kStreamSlack) * 4;
         HIP_TRY(hipMalloc((void **)&d_part, bytes));
@@ -897,7 +977,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     if (int rc = resolve_functions(L)) return rc;
     if (I) {
         I->tile_size_x = x; I->tile_size_y = panel_rows; I->n_col_tiles = n_tiles_all;
-        I->n_row_panels = n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
+        I->n_row_panels = panel_local ? shares : n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
         I->grid = L.grid; I->block = L.block; I->k_slice = ks;
     }
     c.P->info.padded_positions += np;

@@ -261,7 +261,21 @@ void sddmm_tile_kernel(const TileArgs a)
             const int rows = min(a.tile_x, a.n_cols - tile_base);
             const float4 *src = H4 + (size_t)tile_base * row_k4;
             const int n4 = rows * K4;
-            for (int i = threadIdx.x; i < n4; i += NW * 64) {
+            // (eight loads in flight per lane: a workgroup with many tiles in its turn -- a wide matrix --
+            // spends its time between tiles waiting for these, one memory latency per round)
+            constexpr int kStageUnroll = 8, kStride = NW * 64;
+            int i = threadIdx.x;
+            for (; i + (kStageUnroll - 1) * kStride < n4; i += kStageUnroll * kStride) {
+                float4 v[kStageUnroll];
+#pragma unroll
+                for (int u = 0; u < kStageUnroll; ++u) {
+                    const int ii = i + u * kStride, r = ii / K4, q = ii - r * K4;
+                    v[u] = src[(size_t)r * row_k4 + q];
+                }
+#pragma unroll
+                for (int u = 0; u < kStageUnroll; ++u) lds_tile[i + u * kStride] = v[u];
+            }
+            for (; i < n4; i += kStride) {
                 const int r = i / K4, q = i - r * K4;
                 lds_tile[i] = src[(size_t)r * row_k4 + q];
             }
@@ -347,19 +361,15 @@ void sddmm_tile_kernel(const TileArgs a)
         const bool to_part = PART && a.to_part != 0;  // (uniform)
         // (gather form: a position whose index carries bit 31 is padding that worked on
         // another row's column; its result goes to a scratch line instead of the output)
+        // (one store whose address is selected, not a branch around two stores: a branch inside the
+        // loop body costs the later slices of a sliced launch 8 % -- 736 against 679 us on the recommender)
         auto flush = [&]() {
-            if constexpr (PART) {
-                if (to_part) {  // (a padding position has a slot of its own)
-                    *reinterpret_cast<float *>(part_b + pend_o) = pend_v;
-                    return;
-                }
-            }
-            if constexpr (GATHER) {
-                float *dst = (int32_t)pend_p < 0 ? a.sink + (((blockIdx.x & 255) << 6) + lane) : a.out + pend_p;
-                *dst = pend_v;
-            } else {
-                a.out[pend_p] = pend_v;
-            }
+            float *dst;
+            if constexpr (GATHER) dst = (int32_t)pend_p < 0 ? a.sink + (((blockIdx.x & 255) << 6) + lane) : a.out + pend_p;
+            else dst = a.out + pend_p;
+            // (a padding position has a slot of its own in a.part)
+            if constexpr (PART) dst = to_part ? reinterpret_cast<float *>(part_b + pend_o) : dst;
+            *dst = pend_v;
         };
         // c[I]: where the H row this lane works on in step I starts (LDS: byte address of
         // this lane's first piece; gather form: float4 index of the row); cn: the same for the next batch, requested here after the last LDS

@@ -150,6 +150,30 @@ def test_padded_gather_over_column_slabs(oracle, K, slab, panel):
     residual_ok(out2.cpu().numpy(), d, oracle, K)
 
 
+@pytest.mark.parametrize("K", [128, 256])
+def test_banded_rows_walked_by_groups_of_workgroups(oracle, K):
+    """More column tiles than workgroups and rows that touch a dozen tiles each: the rows are cut into ranges, each
+    walked by a group of workgroups of one die (tile_runs = 2).  Checked against the oracle like the plan with whole
+    tiles handed out in runs of neighbours (tile_runs = 1); the two differ in the last bits where a run's short last
+    chunk lands in a batch of the other kind (the items end elsewhere), never by more than a few ulps of the sum."""
+    d = synth.banded(n=16384, per_row=24, half_band=96, K=K, seed=21)
+    outs = {}
+    for runs in (1, 2):
+        plan = host_plan(d, K, kernel=capi.KERNEL_LDS_TILE, tile_size_x=16, tile_runs=runs)
+        info = plan.info()
+        assert info["kernel"] == capi.KERNEL_LDS_TILE and info["n_col_tiles"] == 1024
+        assert (info["n_row_panels"] > 1) == (runs == 2), info
+        dev = torch.device(DEV)
+        W = d["W"].to(dev); H = d["H"].to(dev); out = torch.full((d["nnz"],), float("nan"), device=dev)
+        plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+        outs[runs] = out.cpu()
+    check(d, outs[1].numpy(), oracle, K)
+    check(d, outs[2].numpy(), oracle, K)
+    scale = float(np.abs(outs[1].numpy()).max())
+    assert float((outs[1] - outs[2]).abs().max()) <= 1e-5 * scale
+
+
 def test_concurrent_executes_on_one_plan_and_concurrent_plan_creation(oracle):
     """The header's promise: a plan is immutable, sddmm_execute may be called from several threads on the same plan
     (each on its own stream, outputs apart); plans may also be built concurrently."""
