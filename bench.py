@@ -169,6 +169,8 @@ def main():
                     help="load the plan from PATH.k<K> when that file fits this matrix, K and options; otherwise build it and save it there")
     ap.add_argument("--tile-sweep", action="store_true", help="one row per tile configuration (see the module docstring)")
     ap.add_argument("--from-prof", default=None, metavar="DIR", help="merge a rocprofv3 profile of this workload into the line")
+    ap.add_argument("--fused", action="store_true",
+                    help="also time the forms around the SDDMM on the same workload: row softmax of out, SDDMM + softmax, SpMM")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 1 GiB device copy (a known-size reference for HBM counters)")
     args = ap.parse_args()
@@ -303,6 +305,36 @@ def main():
     }
     if parity is not None:
         line["parity"] = parity
+    if args.fused:
+        # the callers' forms around the SDDMM, on the same matrix and rank: each timed like a step (HIP events on the
+        # launch stream); algorithmic bytes: softmax reads and writes every entry once (8 nnz + the row pointers);
+        # SpMM reads the pattern and its weights (8 nnz), the row pointers and the touched H rows and writes Y
+        set_rank(K0)
+        n_steps, n_warm = max(10, args.steps // 10), max(3, args.warmup // 10)
+        x = torch.empty(d["nnz"], device=dev); y = torch.empty(d["nnz"], device=dev)
+        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(), d["col_ind"].data_ptr(), K0,
+                                         options=capi.PlanOptions.defaults(kernel=kernel, **opt_fields))
+        plan.set_values(d["val"].data_ptr(), torch.cuda.current_stream().cuda_stream)
+        plan.execute(0, d["W"].data_ptr(), d["H"].data_ptr(), x.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        rp, ci = d["row_ptr"].data_ptr(), d["col_ind"].data_ptr()
+        _, sm_ms, _ = time_steps(lambda st: capi.row_softmax(d["n_rows"], rp, x.data_ptr(), y.data_ptr(), st), n_steps, n_warm, torch, 30.0)
+        _, es_ms, _ = time_steps(lambda st: plan.execute_softmax(0, d["W"].data_ptr(), d["H"].data_ptr(), y.data_ptr(), st),
+                                 n_steps, n_warm, torch, 30.0)
+        Y = torch.empty(d["n_rows"], K0, device=dev)
+        _, sp_ms, _ = time_steps(lambda st: capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp, ci, y.data_ptr(), K0,
+                                                          d["H"].data_ptr(), Y.data_ptr(), st), n_steps, n_warm, torch, 30.0)
+        plan.close()
+        sm_bytes = 8.0 * d["nnz"] + 4.0 * (d["n_rows"] + 1)
+        sp_bytes = 8.0 * d["nnz"] + 4.0 * (d["n_rows"] + 1) + 4.0 * K0 * (info["cols_touched"] + d["n_rows"])
+        line["fused"] = {
+            "row_softmax": {"ms": round(sm_ms, 4), "alg_bytes": sm_bytes, "alg_gbps": round(sm_bytes / (sm_ms * 1e6), 1),
+                            "hbm_frac": round(sm_bytes / (sm_ms * 1e6) / HBM_PEAK_GBPS, 4)},
+            "sddmm_plus_softmax": {"ms": round(es_ms, 4)},
+            "spmm_csr": {"ms": round(sp_ms, 4), "gflops": round(2.0 * d["nnz"] * K0 / (sp_ms * 1e6), 1), "alg_bytes": sp_bytes,
+                         "alg_gbps": round(sp_bytes / (sp_ms * 1e6), 1), "hbm_frac": round(sp_bytes / (sp_ms * 1e6) / HBM_PEAK_GBPS, 4)},
+            "steps": n_steps}
+        del x, y, Y
     if args.tile_sweep:
         # tile width x K slice x lanes per nonzero, explicit values honoured by the planner; fewer steps per row
         rows = []

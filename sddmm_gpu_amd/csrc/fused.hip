@@ -10,90 +10,336 @@ using namespace sddmm;
 
 namespace {
 
-__device__ __forceinline__ float wave_max(float v)
+// Row softmax in three kernels over equal chunks of the entries (not of the rows: a matrix may hold a few
+// rows of a million entries next to millions of rows of ten).  The first finds the rows at the ends of every chunk.  In the second a workgroup takes
+// kSmChunk consecutive entries into LDS and gives each of their rows to a lane, a group of lanes, a wave or
+// all its waves, by the row's length: maximum, sum of
+// exponentials, normalisation, all inside LDS; the chunk goes back to memory in one coalesced pass.  A row
+// that reaches beyond the chunk cannot be normalised yet: its piece is stored as exp(x - m) with the
+// piece's own maximum m, and (m, sum) goes into a record of the chunk.  The third kernel visits the chunks
+// again, merges the records of each cut row (at most two per chunk: the row that began before the chunk
+// and the row that ends after it) and scales the stored pieces.  Both kernels read the number of entries
+// from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.
+constexpr int kSmChunk = 4096;
+constexpr int kSmBlock = 256;
+constexpr int kSmRowsMax = kSmChunk + 128;  // row pointers of a chunk kept in LDS at a time
+constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
+
+// (m, sum) of the cut pieces: [2c] the row that began before chunk c, [2c + 1] the row that ends after
+// it.  8 + 4 MiB per device, held until the process ends; kernels name the arrays directly.  Softmax calls that
+// overlap in time on one device share it and must not (calls on one stream never do).
+static __device__ __align__(256) float2 g_softmax_rec[2 * kSmMaxChunks];
+static __device__ __align__(256) int2 g_softmax_rows[kSmMaxChunks];  // first and last row of each chunk
+
+// First kernel: the first and the last row of every chunk, one thread per chunk (two binary searches of
+// row_ptr whose loads the other threads' searches hide).
+__global__ __launch_bounds__(256)
+void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows)
+{
+    const int64_t nnz = row_ptr[n_rows];
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t p0 = c * kSmChunk, p1 = min(nnz, p0 + kSmChunk) - 1;
+        // first row whose end lies beyond p0 / p1
+        int64_t lo0 = 0, hi0 = n_rows - 1, lo1 = 0, hi1 = n_rows - 1;
+        while (lo0 < hi0 || lo1 < hi1) {
+            if (lo0 < hi0) { const int64_t mid = (lo0 + hi0) >> 1; if (row_ptr[mid + 1] <= p0) lo0 = mid + 1; else hi0 = mid; }
+            if (lo1 < hi1) { const int64_t mid = (lo1 + hi1) >> 1; if (row_ptr[mid + 1] <= p1) lo1 = mid + 1; else hi1 = mid; }
+        }
+        g_softmax_rows[c] = make_int2((int)lo0, (int)lo1);
+    }
+}
+
+// exp(x) for x <= 0 in six instructions: 2^t with t = x log2(e) rounded, times 1 + (what the rounding of t
+// and of log2(e) left out) ln 2.  About one ulp; the library routine costs four times as much, and these
+// passes would be bound by it.
+__device__ __forceinline__ float exp_nonpositive(float x)
+{
+    const float l2e = 1.44269502e+0f, l2e_lo = 1.92596299e-8f;
+    const float t = x * l2e;
+    const float r = fmaf(x, l2e_lo, fmaf(x, l2e, -t));
+    const float e = __builtin_amdgcn_exp2f(t);
+    return fmaf(e, r * 0.693147182f, e);
+}
+
+template <int GW>
+__device__ __forceinline__ float group_max(float v)
 {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    for (int off = GW / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
     return v;
 }
-__device__ __forceinline__ float wave_sum(float v)
+template <int GW>
+__device__ __forceinline__ float group_sum(float v)
 {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    for (int off = GW / 2; off > 0; off >>= 1) v += __shfl_xor(v, off);
     return v;
 }
 
-// Row softmax, one wave per row up to kLongRow entries: the row is read once (up to 8 entries per
-// lane stay in registers between the passes), longer rows are read three times by a whole workgroup.
-constexpr int kSoftmaxBlock = 256;
-constexpr int kRegs = 8;                   // entries per lane kept in registers: rows up to 512 entries
-constexpr int kLongRow = 64 * kRegs;
+// One row's piece buf[b, e) of a chunk: exp(x - max) in place and the sum; a whole row is normalised, a cut
+// row leaves (max, sum) in *rec.  Four forms, by how many lanes work on the row.
 
-__global__ __launch_bounds__(kSoftmaxBlock)
-void sddmm_row_softmax_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out)
+// one lane (rows of a few entries: no lane exchanges at all)
+__device__ __forceinline__ void softmax_piece_by_lane(float *buf, int b, int e, bool whole, float2 *rec)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t wave = ((int64_t)blockIdx.x * kSoftmaxBlock + threadIdx.x) >> 6;
-    const int64_t n_waves = ((int64_t)gridDim.x * kSoftmaxBlock) >> 6;
-    for (int64_t r = wave; r < n_rows; r += n_waves) {
-        const int b = row_ptr[r], e = row_ptr[r + 1];
-        const int n = e - b;
-        if (n <= 0 || n > kLongRow) continue;  // long rows: the other kernel
-        float v[kRegs];
-        float mx = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            const int p = b + lane + 64 * i;
-            v[i] = p < e ? x[p] : -INFINITY;
-            mx = fmaxf(mx, v[i]);
-        }
-        mx = wave_max(mx);
-        float sum = 0.f;
-#pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            v[i] = expf(v[i] - mx);  // exp(-inf) = 0 for the lanes past the row's end
-            sum += v[i];
-        }
-        sum = wave_sum(sum);
+    float m = -INFINITY;
+    for (int i = b; i < e; ++i) m = fmaxf(m, buf[i]);
+    float sum = 0.f;
+    for (int i = b; i < e; ++i) {
+        const float t = exp_nonpositive(buf[i] - m);
+        buf[i] = t;
+        sum += t;
+    }
+    if (whole) {
         const float inv = 1.0f / sum;
+        for (int i = b; i < e; ++i) buf[i] *= inv;
+    } else {
+        *rec = make_float2(m, sum);
+    }
+}
+
+// a group of GW lanes (all of them call this with the same row; the lane exchanges stay inside the group)
+template <int GW>
+__device__ __forceinline__ void softmax_piece_by_group(float *buf, int b, int e, bool whole, float2 *rec)
+{
+    const int gl = threadIdx.x & (GW - 1);
+    // (four independent entries per round, so that the LDS reads of a long row overlap)
+    float m = -INFINITY;
+    int i = b + gl;
+    for (; i + 3 * GW < e; i += 4 * GW)
+        m = fmaxf(fmaxf(m, fmaxf(buf[i], buf[i + GW])), fmaxf(buf[i + 2 * GW], buf[i + 3 * GW]));
+    for (; i < e; i += GW) m = fmaxf(m, buf[i]);
+    m = group_max<GW>(m);
+    float sum = 0.f;
+    i = b + gl;
+    for (; i + 3 * GW < e; i += 4 * GW) {
+        const float t0 = exp_nonpositive(buf[i] - m), t1 = exp_nonpositive(buf[i + GW] - m),
+                    t2 = exp_nonpositive(buf[i + 2 * GW] - m), t3 = exp_nonpositive(buf[i + 3 * GW] - m);
+        buf[i] = t0; buf[i + GW] = t1; buf[i + 2 * GW] = t2; buf[i + 3 * GW] = t3;
+        sum += (t0 + t1) + (t2 + t3);
+    }
+    for (; i < e; i += GW) {
+        const float t = exp_nonpositive(buf[i] - m);
+        buf[i] = t;
+        sum += t;
+    }
+    sum = group_sum<GW>(sum);
+    if (whole) {
+        const float inv = 1.0f / sum;
+        for (i = b + gl; i < e; i += GW) buf[i] *= inv;
+    } else if (gl == 0) {
+        *rec = make_float2(m, sum);
+    }
+}
+
+// the whole workgroup (every thread calls this with the same row).  red: 2 x (waves per workgroup) floats of LDS
+__device__ __forceinline__ void softmax_piece_by_workgroup(float *buf, float *red, int b, int e, bool whole, float2 *rec)
+{
+    constexpr int NW = kSmBlock / 64;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float m = -INFINITY;
+    int i = b + threadIdx.x;
+    for (; i + 3 * kSmBlock < e; i += 4 * kSmBlock)
+        m = fmaxf(fmaxf(m, fmaxf(buf[i], buf[i + kSmBlock])), fmaxf(buf[i + 2 * kSmBlock], buf[i + 3 * kSmBlock]));
+    for (; i < e; i += kSmBlock) m = fmaxf(m, buf[i]);
+    m = group_max<64>(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
 #pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            const int p = b + lane + 64 * i;
-            if (p < e) out[p] = v[i] * inv;
+    for (int w = 0; w < NW; ++w) m = fmaxf(m, red[w]);
+    float sum = 0.f;
+    i = b + threadIdx.x;
+    for (; i + 3 * kSmBlock < e; i += 4 * kSmBlock) {
+        const float t0 = exp_nonpositive(buf[i] - m), t1 = exp_nonpositive(buf[i + kSmBlock] - m),
+                    t2 = exp_nonpositive(buf[i + 2 * kSmBlock] - m), t3 = exp_nonpositive(buf[i + 3 * kSmBlock] - m);
+        buf[i] = t0; buf[i + kSmBlock] = t1; buf[i + 2 * kSmBlock] = t2; buf[i + 3 * kSmBlock] = t3;
+        sum += (t0 + t1) + (t2 + t3);
+    }
+    for (; i < e; i += kSmBlock) {
+        const float t = exp_nonpositive(buf[i] - m);
+        buf[i] = t;
+        sum += t;
+    }
+    sum = group_sum<64>(sum);
+    if (lane == 0) red[NW + wave] = sum;
+    __syncthreads();  // (also: everyone has read the maxima, so the next row may overwrite them)
+    sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[NW + w];
+    if (whole) {
+        const float inv = 1.0f / sum;
+        for (i = b + threadIdx.x; i < e; i += kSmBlock) buf[i] *= inv;
+    } else if (threadIdx.x == 0) {
+        *rec = make_float2(m, sum);
+    }
+    // (the sums are read before the next row's second barrier, which comes after its first: no barrier needed here)
+}
+
+// piece lengths up to which a row is worked on by a lane / a group of 16 lanes / a wave; beyond: the workgroup
+constexpr int kSmByLane = 8, kSmBy16 = 192, kSmByWave = 1023;
+constexpr int kSmList16 = kSmChunk / (kSmByLane + 1) + 1, kSmList64 = kSmChunk / (kSmBy16 + 1) + 1,
+              kSmListWg = kSmChunk / (kSmByWave + 1) + 1;
+
+__global__ __launch_bounds__(kSmBlock)
+void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out)
+{
+    __shared__ __align__(16) float buf[kSmChunk];
+    __shared__ int32_t rows_lds[kSmRowsMax];
+    __shared__ float red[2 * kSmBlock / 64];
+    // rows of the chunk that take more than a lane, by class (index of the row inside the round's window)
+    __shared__ uint16_t list16[kSmList16], list64[kSmList64], list_wg[kSmListWg];
+    __shared__ int n_listed[3];
+    constexpr int kPer = kSmChunk / 4 / kSmBlock;  // float4 per thread and chunk
+    const int64_t nnz = row_ptr[n_rows];
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    // A whole chunk travels memory -> registers -> LDS; the registers are filled one chunk ahead, so the
+    // memory latency of chunk c + grid passes while chunk c is worked on.
+    float4 ahead[kPer];
+    int2 rows_ahead = make_int2(0, 0);
+    auto request = [&](int64_t c) {
+        if (c < n_chunks) rows_ahead = g_softmax_rows[c];
+        if (c < n_chunks && vec_in && (c + 1) * kSmChunk <= nnz) {
+            const float4 *src = reinterpret_cast<const float4 *>(x + c * kSmChunk);
+#pragma unroll
+            for (int u = 0; u < kPer; ++u) ahead[u] = src[threadIdx.x + u * kSmBlock];
+        }
+    };
+    request(blockIdx.x);
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int64_t c0 = c * kSmChunk, c1 = min(nnz, c0 + kSmChunk);
+        const int n = (int)(c1 - c0);
+        __syncthreads();  // the chunk before has left the buffers
+        if (n == kSmChunk && vec_in) {
+#pragma unroll
+            for (int u = 0; u < kPer; ++u) reinterpret_cast<float4 *>(buf)[threadIdx.x + u * kSmBlock] = ahead[u];
+        } else {
+            for (int i0 = threadIdx.x; i0 < n; i0 += 8 * kSmBlock) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = i0 + u * kSmBlock < n ? x[c0 + i0 + u * kSmBlock] : 0.f;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) if (i0 + u * kSmBlock < n) buf[i0 + u * kSmBlock] = v[u];
+            }
+        }
+        const int64_t r0 = rows_ahead.x, r1 = rows_ahead.y;
+        // The chunk's row pointers go into LDS, kSmRowsMax - 1 rows at a time (one round unless the chunk is
+        // full of empty rows).  These loads are issued before the next chunk is requested, so that waiting
+        // for them does not wait for it.
+        for (int64_t w0 = r0; w0 <= r1; w0 += kSmRowsMax - 1) {
+            const int n_w = (int)(min(r1, w0 + kSmRowsMax - 2) - w0 + 1);  // rows of this round
+            if (w0 != r0) __syncthreads();  // the round before has left rows_lds and the lists
+            for (int i = threadIdx.x; i <= n_w; i += kSmBlock) rows_lds[i] = row_ptr[w0 + i];
+            if (threadIdx.x < 3) n_listed[threadIdx.x] = 0;
+            if (w0 == r0) request(c + gridDim.x);
+            __syncthreads();
+            auto piece = [&](int k, int *b, int *e, bool *whole, float2 **rec) {
+                const int64_t rb = rows_lds[k], re = rows_lds[k + 1];
+                *b = (int)(max(rb, c0) - c0); *e = (int)(min(re, c1) - c0);
+                *whole = rb >= c0 && re <= c1;
+                *rec = &g_softmax_rec[2 * c + (rb < c0 ? 0 : 1)];
+            };
+            // every thread looks at the rows k = t, t + 256, ...: the short ones it does itself, the others it lists
+            for (int k = threadIdx.x; k < n_w; k += kSmBlock) {
+                int b, e; bool whole; float2 *rec;
+                piece(k, &b, &e, &whole, &rec);
+                const int len = e - b;
+                if (len <= 0) continue;
+                if (len <= kSmByLane) softmax_piece_by_lane(buf, b, e, whole, rec);
+                else if (len <= kSmBy16) list16[atomicAdd(&n_listed[0], 1)] = (uint16_t)k;
+                else if (len <= kSmByWave) list64[atomicAdd(&n_listed[1], 1)] = (uint16_t)k;
+                else list_wg[atomicAdd(&n_listed[2], 1)] = (uint16_t)k;
+            }
+            __syncthreads();
+            const int n16 = n_listed[0], n64 = n_listed[1], n_wg = n_listed[2];
+            for (int q = 0; q < n_wg; ++q) {
+                int b, e; bool whole; float2 *rec;
+                piece(list_wg[q], &b, &e, &whole, &rec);
+                softmax_piece_by_workgroup(buf, red, b, e, whole, rec);
+            }
+            for (int q = threadIdx.x >> 6; q < n64; q += kSmBlock / 64) {
+                int b, e; bool whole; float2 *rec;
+                piece(list64[q], &b, &e, &whole, &rec);
+                softmax_piece_by_group<64>(buf, b, e, whole, rec);
+            }
+            for (int q = threadIdx.x >> 4; q < n16; q += kSmBlock / 16) {
+                int b, e; bool whole; float2 *rec;
+                piece(list16[q], &b, &e, &whole, &rec);
+                softmax_piece_by_group<16>(buf, b, e, whole, rec);
+            }
+        }
+        __syncthreads();
+        if (n == kSmChunk && vec_out) {
+            float4 *dst = reinterpret_cast<float4 *>(out + c0);
+#pragma unroll
+            for (int u = 0; u < kPer; ++u) dst[threadIdx.x + u * kSmBlock] = reinterpret_cast<const float4 *>(buf)[threadIdx.x + u * kSmBlock];
+        } else {
+            for (int i = threadIdx.x; i < n; i += kSmBlock) out[c0 + i] = buf[i];
         }
     }
 }
 
-// One workgroup per long row (rows listed nowhere: every workgroup scans its share of the rows
-// and takes the long ones it finds; there are few).
-__global__ __launch_bounds__(kSoftmaxBlock)
-void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out)
+// (m, sum) of row [rb, re) from the records of the chunks it spans: the last-slot record of its first
+// chunk, the first-slot records of the others; every wave of the workgroup computes the same pair.
+__device__ __forceinline__ float2 merged_record(int64_t rb, int64_t re)
 {
-    __shared__ float red[kSoftmaxBlock / 64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int64_t r = blockIdx.x; r < n_rows; r += gridDim.x) {
-        const int b = row_ptr[r], e = row_ptr[r + 1];
-        if (e - b <= kLongRow) continue;
-        float mx = -INFINITY;
-        for (int p = b + threadIdx.x; p < e; p += kSoftmaxBlock) mx = fmaxf(mx, x[p]);
-        mx = wave_max(mx);
-        __syncthreads();
-        if (lane == 0) red[wave] = mx;
-        __syncthreads();
-        mx = red[0];
+    const int lane = threadIdx.x & 63;
+    const int64_t ca = rb / kSmChunk, cb = (re - 1) / kSmChunk;
+    float m = -INFINITY, s = 0.f;
+    for (int64_t k = ca + lane; k <= cb; k += 64) {
+        const float2 rec = g_softmax_rec[2 * k + (k == ca ? 1 : 0)];
+        const float mn = fmaxf(m, rec.x);
+        s = s * expf(m - mn) + rec.y * expf(rec.x - mn);  // (exp(-inf - finite) = 0 for the first record)
+        m = mn;
+    }
 #pragma unroll
-        for (int w = 1; w < kSoftmaxBlock / 64; ++w) mx = fmaxf(mx, red[w]);
-        float sum = 0.f;
-        for (int p = b + threadIdx.x; p < e; p += kSoftmaxBlock) sum += expf(x[p] - mx);
-        sum = wave_sum(sum);
-        __syncthreads();
-        if (lane == 0) red[wave] = sum;
-        __syncthreads();
-        sum = 0.f;
+    for (int off = 32; off > 0; off >>= 1) {
+        const float m2 = __shfl_xor(m, off), s2 = __shfl_xor(s, off);
+        const float mn = fmaxf(m, m2);
+        // (a lane without records holds (-inf, 0): its term must vanish without producing inf - inf)
+        const float t1 = m == -INFINITY ? 0.f : s * expf(m - mn), t2 = m2 == -INFINITY ? 0.f : s2 * expf(m2 - mn);
+        s = t1 + t2;
+        m = mn;
+    }
+    return make_float2(m, s);
+}
+
+// out[b..e) *= f by the whole workgroup, eight entries per thread in flight
+__device__ __forceinline__ void scale_range(float *out, int64_t b, int64_t e, float f)
+{
+    for (int64_t i0 = b + threadIdx.x; i0 < e; i0 += 8 * kSmBlock) {
+        float v[8];
 #pragma unroll
-        for (int w = 0; w < kSoftmaxBlock / 64; ++w) sum += red[w];
-        const float inv = 1.0f / sum;
-        for (int p = b + threadIdx.x; p < e; p += kSoftmaxBlock) out[p] = expf(x[p] - mx) * inv;
+        for (int u = 0; u < 8; ++u) v[u] = i0 + u * kSmBlock < e ? out[i0 + u * kSmBlock] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) if (i0 + u * kSmBlock < e) out[i0 + u * kSmBlock] = v[u] * f;
+    }
+}
+
+__global__ __launch_bounds__(kSmBlock)
+void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, float *out)
+{
+    const int64_t nnz = row_ptr[n_rows];
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const int64_t c0 = c * kSmChunk, c1 = min(nnz, c0 + kSmChunk);
+        const int2 rr = g_softmax_rows[c];
+        const int64_t r0 = rr.x, r1 = rr.y;
+        const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
+        if (b0 < c0 || e0 > c1) {  // the chunk's first row is cut (it began before the chunk, or it fills it and goes on)
+            const float2 all = merged_record(b0, e0);
+            const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
+            const float f = expf(mine.x - all.x) / all.y;
+            const int64_t pb = max(b0, c0), pe = min(e0, c1);
+            scale_range(out, pb, pe, f);
+        }
+        if (r1 != r0 && e1 > c1) {  // another row begins inside the chunk and ends after it
+            const float2 all = merged_record(b1, e1);
+            const float2 mine = g_softmax_rec[2 * c + 1];
+            const float f = expf(mine.x - all.x) / all.y;
+            scale_range(out, b1, c1, f);
+        }
     }
 }
 
@@ -223,11 +469,11 @@ namespace sddmm {
 int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream)
 {
     if (n_rows <= 0) return SDDMM_OK;
-    const unsigned grid = (unsigned)std::min<int64_t>((n_rows * 64 + kSoftmaxBlock - 1) / kSoftmaxBlock, 256 * 64);
-    hipLaunchKernelGGL(sddmm_row_softmax_kernel, dim3(grid), dim3(kSoftmaxBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out);
-    const unsigned grid_long = (unsigned)std::min<int64_t>(n_rows, 256 * 8);
-    hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(grid_long), dim3(kSoftmaxBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows,
-                       d_x, d_out);
+    // (the entry count lives on the device: the grid is sized for the machine, the kernels stride over the chunks)
+    const unsigned grid = 256 * 4;  // (33 KB of LDS per workgroup: four per compute unit)
+    hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out);
+    hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out);
     return last_error("sddmm_row_softmax");
 }
 
@@ -238,6 +484,7 @@ extern "C" {
 int sddmm_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream)
 {
     if (n_rows < 0 || (n_rows > 0 && (!d_row_ptr || !d_x || !d_out))) return fail(SDDMM_ERR_ARG, "sddmm_row_softmax: bad arguments");
+    if (n_rows >= INT32_MAX) return fail(SDDMM_ERR_RANGE, "sddmm_row_softmax: more than 2^31 - 2 rows");
     return launch_row_softmax(n_rows, d_row_ptr, d_x, d_out, stream);
 }
 

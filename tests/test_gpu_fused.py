@@ -39,18 +39,31 @@ def test_row_softmax_matches_oracle(oracle, cfg, scale):
     assert np.allclose(ones.cpu().numpy(), 1.0 / deg[d["row_ind"].numpy()], rtol=1e-6, atol=0)
 
 
-def test_row_softmax_edge_rows(oracle):
-    # empty rows, rows of 1, 64, 65, 512, 513 and 5000 entries (the register path ends at 512)
-    lens = [0, 1, 0, 64, 65, 512, 513, 5000, 0, 2, 511]
+@pytest.mark.parametrize("misalign", [0, 1])
+def test_row_softmax_edge_rows(oracle, misalign):
+    """Rows at the boundaries of the kernel's cases: entries are worked on in chunks of 4096; inside a chunk a row goes to
+    a lane (up to 8 entries), 16 lanes (up to 192), a wave (up to 1023) or the workgroup; a row cut by a chunk boundary is
+    finished by a second pass over the records of its pieces; a chunk's row pointers are staged 4223 rows at a time."""
+    lens = ([0, 1, 0, 8, 9, 64, 65, 192, 193, 1023, 1024, 0, 2, 511]      # every class, whole rows
+            + [4096 - sum([1, 8, 9, 64, 65, 192, 193, 1023, 1024, 2, 511])]  # ... up to the end of chunk 0 exactly
+            + [4096]                                                        # a row that is exactly chunk 1
+            + [5000, 3]                                                     # a row over two chunk boundaries, then a short one
+            + [0] * 6000 + [1, 2] * 700 + [0] * 5000                        # runs of empty rows longer than a staging round
+            + [13000]                                                       # a row over three boundaries with whole chunks inside
+            + [2] * 3000 + [7, 0, 300, 5])
     rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     rng = np.random.default_rng(1)
     x = rng.normal(0, 10, rp[-1]).astype(np.float32)
-    x[rp[5]] = 80.0; x[rp[7] + 17] = -90.0
+    x[rp[5]] = 80.0; x[rp[lens.index(5000)] + 17] = -90.0; x[rp[lens.index(13000)] + 12000] = 75.0
     dev = torch.device(DEV)
-    xd = torch.from_numpy(x).to(dev); out = torch.full_like(xd, float("nan"))
+    # (misalign: x and out start 4 bytes past a 16-byte boundary, which takes the kernels' scalar load/store path)
+    xbuf = torch.zeros(len(x) + 4, device=dev); obuf = torch.full((len(x) + 4,), float("nan"), device=dev)
+    xd = xbuf[misalign:misalign + len(x)]; out = obuf[misalign:misalign + len(x)]
+    xd.copy_(torch.from_numpy(x))
     capi.row_softmax(len(lens), torch.from_numpy(rp).to(dev).data_ptr(), xd.data_ptr(), out.data_ptr())
     torch.cuda.synchronize()
     softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
+    assert bool(torch.isnan(obuf[:misalign]).all()) and bool(torch.isnan(obuf[misalign + len(x):]).all())  # nothing written outside
     capi.row_softmax(0, 0, 0, 0)  # nothing to do
 
 
