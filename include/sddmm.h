@@ -329,9 +329,13 @@ int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const flo
  * row-wise softmax of the results in place:
  *   out[p] = exp(s_p - m_r) / sum_{q in row r} exp(s_q - m_r),  s = val .* (W H^T) on S's pattern,
  * m_r the row's largest s.  One extra pass over out (the row totals must be known
- * before any entry can be normalised); rows up to 512 entries are read once.
+ * before any entry can be normalised), made in equal chunks of entries whatever
+ * the rows' lengths; a row cut by a chunk boundary is finished from per-chunk
+ * (max, sum) records kept in a fixed device array of the library (12 MiB per
+ * GPU), so softmax calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream never do.
  * sddmm_row_softmax: the same pass on its own, over any CSR pattern in device
- * memory (d_out may be d_x).
+ * memory (d_out may be d_x; n_rows < 2^31 - 1, row_ptr[n_rows] entries).
  * sddmm_spmm_csr: Y[r, 0:K] = sum over row r's entries p of x[p] * H[col_p, 0:K]
  * (d_Y: n_rows*K fp32, overwritten; rows without entries become 0), the product
  * that consumes the attention weights.  Rows that straddle the 256-entry chunks
