@@ -65,6 +65,10 @@ def test_row_softmax_edge_rows(oracle, misalign):
     softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
     assert bool(torch.isnan(obuf[:misalign]).all()) and bool(torch.isnan(obuf[misalign + len(x):]).all())  # nothing written outside
     capi.row_softmax(0, 0, 0, 0)  # nothing to do
+    empty_rp = torch.zeros(6, dtype=torch.int32, device=dev)  # five rows, no entries
+    capi.row_softmax(5, empty_rp.data_ptr(), xd.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(obuf[:misalign]).all())  # (and nothing was written)
 
 
 @pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])

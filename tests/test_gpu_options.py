@@ -151,7 +151,7 @@ def test_padded_gather_over_column_slabs(oracle, K, slab, panel):
 
 
 @pytest.mark.parametrize("K", [128, 256])
-def test_banded_rows_walked_by_groups_of_workgroups(oracle, K):
+def test_banded_rows_walked_by_groups_of_workgroups(oracle, tmp_path, K):
     """More column tiles than workgroups and rows that touch a dozen tiles each: the rows are cut into ranges, each
     walked by a group of workgroups of one die (tile_runs = 2).  Checked against the oracle like the plan with whole
     tiles handed out in runs of neighbours (tile_runs = 1); the two differ in the last bits where a run's short last
@@ -172,6 +172,22 @@ def test_banded_rows_walked_by_groups_of_workgroups(oracle, K):
     check(d, outs[2].numpy(), oracle, K)
     scale = float(np.abs(outs[1].numpy()).max())
     assert float((outs[1] - outs[2]).abs().max()) <= 1e-5 * scale
+    # the same without short batches (the other stream layout), and through a plan file
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    o = capi.PlanOptions.defaults(ignore_env=1, kernel=capi.KERNEL_LDS_TILE, tile_size_x=16, tile_runs=2, tile_short_batches=0)
+    plan = S.plan(K, options=o)
+    assert plan.info()["n_row_panels"] > 1 and plan.info()["short_batches"] == 0
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev); out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    check(d, out.cpu().numpy(), oracle, K)
+    plan.save(tmp_path / "banded.plan")
+    loaded = S.load_plan(tmp_path / "banded.plan", K, options=o)
+    out2 = torch.full_like(out, float("nan"))
+    loaded.execute(0, W.data_ptr(), H.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
 
 
 def test_concurrent_executes_on_one_plan_and_concurrent_plan_creation(oracle):
