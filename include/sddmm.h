@@ -240,6 +240,8 @@ typedef struct sddmm_plan_options {
     int32_t dense_blocks;       /* 0/1 dense core on the matrix cores (-1: by K)    [SDDMM_DENSE]         */
     int32_t dense_permille;     /* least fill of a dense block, in 1/1000           [SDDMM_DENSE_PERMILLE] */
     int32_t dense_rb_group;     /* row blocks swept together by one die             [SDDMM_DENSE_RB_GROUP] */
+    int32_t fuse_slices;        /* 0/1 the K slices of a launch run inside one kernel
+                                   launch (-1: where the stream is small)           [SDDMM_FUSE_SLICES]   */
     int32_t ignore_env;         /* 1: the environment is not consulted                                      */
     int64_t gather_slab_cols;   /* padded gather streams S in slabs of this many columns [SDDMM_GATHER_SLAB_COLS] */
     int64_t gather_panel_rows;  /* ... and, inside, in panels of this many listed rows   [SDDMM_GATHER_PANEL_ROWS] */

@@ -44,7 +44,7 @@ class PlanOptions(C.Structure):
     _fields_ = [(n, c_int32) for n in (
         "kernel", "tile_size_x", "tile_size_y", "k_slice", "tile_lanes", "tile_waves", "tile_assign", "tile_few_blocks",
         "tile_short_batches", "tile_deal", "tile_runs", "gather_lanes", "gather_padded", "gather_sink", "row_padded",
-        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "ignore_env")] + [(n, c_int64) for n in (
+        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "fuse_slices", "ignore_env")] + [(n, c_int64) for n in (
         "gather_slab_cols", "gather_panel_rows", "dense_min_nnz", "panel_bytes", "short_row_max", "stage_factor", "split_min_nnz")]
 
     @classmethod

@@ -39,8 +39,9 @@ struct Launch {
     KernelFn fn = nullptr;   // stream kernels
     PanelFn pfn = nullptr;   // panel kernel
     TileFn tfn = nullptr;        // tile kernel (values in stream order, first K slice); null: not a tile launch
-    TileFn tfns[5][3] = {};      // [values in stream order / in sorted order / none / residual epilogue with values
-                                 //  in stream order / in sorted order][the only K slice / first of several / a later one]
+    TileFn tfns[5][4] = {};      // [values in stream order / in sorted order / none / residual epilogue with values
+                                 //  in stream order / in sorted order][the only K slice / first of several / a later one /
+                                 //  all slices inside one launch (null: no such variant)]
     KArgs ka{};
     PanelArgs pa{};
     TileArgs ta{};
@@ -54,6 +55,7 @@ struct Launch {
     // what the function pointers above were looked up with (they are looked up again when a saved plan is loaded)
     int32_t fn_kind = 0;  // 1 stream kernel (row gather), 2 stream kernel with an LDS tile, 3 tile kernel, 4 panel, 5 dense
     int32_t fn_g = 0, fn_kpl = 0, fn_exact = 0, fn_gather = 0, fn_nwaves = 0;
+    int32_t fused_slices = 0;  // sliced tile launch small enough that its K slices run inside one kernel launch
 };
 
 struct sddmm_plan {
@@ -193,7 +195,7 @@ void default_options(sddmm_plan_options &o)
     o.kernel = SDDMM_KERNEL_AUTO;
     o.tile_size_x = 0; o.tile_size_y = 0;
     o.k_slice = -1; o.tile_lanes = -1; o.tile_waves = -1; o.tile_assign = -1; o.tile_few_blocks = -1;
-    o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.gather_lanes = -1; o.gather_padded = -1;
+    o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.fuse_slices = -1; o.gather_lanes = -1; o.gather_padded = -1;
     o.gather_sink = -1; o.row_padded = -1; o.unpadded_tile = -1; o.dense_blocks = -1; o.dense_permille = -1;
     o.dense_rb_group = -1; o.ignore_env = 0;
     o.gather_slab_cols = -1; o.gather_panel_rows = -1; o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
@@ -208,7 +210,7 @@ void apply_env_overrides(sddmm_plan_options &o)
     i32("SDDMM_KERNEL", o.kernel); i32("SDDMM_TILE_X", o.tile_size_x); i32("SDDMM_TILE_Y", o.tile_size_y);
     i32("SDDMM_TILE_KSLICE", o.k_slice); i32("SDDMM_TILE_G", o.tile_lanes); i32("SDDMM_TILE_WAVES", o.tile_waves);
     i32("SDDMM_TILE_ASSIGN", o.tile_assign); i32("SDDMM_TILE_FEW_BLOCKS", o.tile_few_blocks);
-    i32("SDDMM_TILE_SHORT", o.tile_short_batches); i32("SDDMM_TILE_DEAL", o.tile_deal); i32("SDDMM_TILE_RUNS", o.tile_runs);
+    i32("SDDMM_TILE_SHORT", o.tile_short_batches); i32("SDDMM_TILE_DEAL", o.tile_deal); i32("SDDMM_TILE_RUNS", o.tile_runs); i32("SDDMM_FUSE_SLICES", o.fuse_slices);
     i32("SDDMM_GATHER_G", o.gather_lanes); i32("SDDMM_GATHER_PADDED", o.gather_padded); i32("SDDMM_GATHER_SINK", o.gather_sink);
     i32("SDDMM_ROW_PADDED", o.row_padded); i32("SDDMM_UNPADDED_TILE", o.unpadded_tile); i32("SDDMM_DENSE", o.dense_blocks);
     i32("SDDMM_DENSE_PERMILLE", o.dense_permille); i32("SDDMM_DENSE_RB_GROUP", o.dense_rb_group);
@@ -234,8 +236,9 @@ int resolve_functions(Launch &L)
     case 3: {
         const TileVariant tv{L.fn_g, L.fn_kpl};
         for (int vm = 0; vm < 5; ++vm)
-            for (int ac = 0; ac < 3; ++ac) {
+            for (int ac = 0; ac < 4; ++ac) {
                 L.tfns[vm][ac] = tile_kernel(tv, vm, L.fn_gather != 0, ac, L.fn_nwaves);
+                if (!L.tfns[vm][ac] && ac == 3) { L.fused_slices = 0; continue; }  // (that form exists for some variants only)
                 if (!L.tfns[vm][ac]) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for lanes %d x %d", tv.G, tv.KPL);
                 HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][ac], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
             }
@@ -957,6 +960,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         c.P->owned.push_back({d_part, bytes, true});
         c.dev_bytes += (int64_t)bytes;
         a.part = d_part;
+        // A small launch costs about as much as its work: its K slices then run inside one kernel launch, every wave
+        // over its own positions slice after slice (K=256, ms per step: bag-of-words 0.0328 -> 0.0309; recommender
+        // shape at 1.1 M nonzeros 0.0381 -> 0.0345, at 5.3 M 0.1267 -> 0.1218).  Not for large streams, whose
+        // workgroups share W rows in L2 by being on the same slice at the same time (99.8 M: 1.710 -> 1.742).
+        L.fused_slices = c.opt.fuse_slices >= 0 ? (c.opt.fuse_slices != 0) : (np <= ((int64_t)1 << 23));
     }
     if (gather) {
         float *d_sink = nullptr;
@@ -1359,7 +1367,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         if (int rc = c.need_row_ptr()) return rc;
     if (!P->launches.empty() && I.grid == 0) { I.grid = P->launches[0].grid; I.block = P->launches[0].block; I.lds_bytes = P->launches[0].lds; }
     I.n_launches = 0;
-    for (const Launch &L : P->launches) I.n_launches += (L.k_slice > 0 && L.k_slice < K) ? K / L.k_slice : 1;
+    for (const Launch &L : P->launches) I.n_launches += (L.k_slice > 0 && L.k_slice < K && !L.fused_slices) ? K / L.k_slice : 1;
     I.device_bytes = c.dev_bytes;
     I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     guard.p = nullptr;
@@ -1509,6 +1517,10 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
         const int vm = residual ? (ta.sval ? 3 : 4) : ta.sval ? 0 : (val ? 1 : 2);
         const bool sliced = L.k_slice < I.K;
+        if (sliced && L.fused_slices) {
+            ta.k_off = 0; ta.n_slices = I.K / L.k_slice; ta.to_part = 0;
+            hipLaunchKernelGGL(L.tfns[vm][3], dim3((unsigned)L.grid), dim3((unsigned)L.block), (size_t)L.lds, stream, ta);
+        } else
         for (int k_off = 0; k_off < I.K; k_off += L.k_slice) {
             ta.k_off = k_off;
             ta.to_part = sliced && k_off + L.k_slice < I.K;
@@ -1645,7 +1657,7 @@ bool same_options(const sddmm_plan_options &a, const sddmm_plan_options &b)
     const int la = a.tile_lanes < 0 ? 0 : a.tile_lanes, lb = b.tile_lanes < 0 ? 0 : b.tile_lanes;
     return a.kernel == b.kernel && a.tile_size_x == b.tile_size_x && a.tile_size_y == b.tile_size_y && a.k_slice == b.k_slice &&
            la == lb && a.tile_waves == b.tile_waves && a.tile_assign == b.tile_assign && a.tile_few_blocks == b.tile_few_blocks &&
-           a.tile_short_batches == b.tile_short_batches && a.tile_deal == b.tile_deal && a.tile_runs == b.tile_runs &&
+           a.tile_short_batches == b.tile_short_batches && a.tile_deal == b.tile_deal && a.tile_runs == b.tile_runs && a.fuse_slices == b.fuse_slices &&
            a.gather_lanes == b.gather_lanes && a.gather_padded == b.gather_padded && a.gather_sink == b.gather_sink &&
            a.row_padded == b.row_padded && a.unpadded_tile == b.unpadded_tile && a.dense_blocks == b.dense_blocks &&
            a.dense_permille == b.dense_permille && a.dense_rb_group == b.dense_rb_group &&
@@ -1923,7 +1935,7 @@ int sddmm_execute_profiled(const sddmm_plan *plan, const float *d_val, const flo
         prof[i].kernel = L.kind;
         prof[i].lanes_per_nnz = L.dfn ? 0 : L.kind == SDDMM_KERNEL_PANEL ? 8 : (L.tfn ? L.tile_g : L.gather_g);
         prof[i].k_slice = L.k_slice;
-        prof[i].n_kernel_launches = (L.k_slice > 0 && L.k_slice < plan->info.K) ? plan->info.K / L.k_slice : 1;
+        prof[i].n_kernel_launches = (L.k_slice > 0 && L.k_slice < plan->info.K && !L.fused_slices) ? plan->info.K / L.k_slice : 1;
         prof[i].nnz = L.nnz;
         prof[i].rows = L.rows;
         prof[i].stream_positions = L.positions;

@@ -84,6 +84,7 @@ struct TileArgs {
     int32_t tile_x, n_cols;
     int32_t K;           // row length of W and H
     int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)
+    int32_t n_slices;    // the all-slices-in-one-launch form: K slices walked inside the launch, from k_off on
 };
 struct TileVariant {
     int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL

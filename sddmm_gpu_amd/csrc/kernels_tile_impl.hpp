@@ -162,10 +162,15 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // results go to a.part, in stream order: one coalesced store per batch); 2 = a later slice (adds to the
 // partial result read back from a.part, coalesced, and stores to a.part again or, in the last slice,
 // a.to_part == 0, to out).  Only the last slice touches out, with one scattered store per position.
+// 3 = all a.n_slices K slices inside this one launch, one after the other (small matrices, where a
+// launch costs as much as its work): a wave meets the same positions in every slice, so the partial
+// results it left in a.part are its own, and a workgroup barrier between the slices is all the
+// ordering needed.
 template <int G, int KPL, int VMODE, int NW, bool GATHER, int SLICE>
 __global__ __launch_bounds__(NW * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
+    constexpr bool FUSED = SLICE == 3;
     constexpr bool ACC = SLICE == 2;
     constexpr bool PART = SLICE >= 1;
     extern __shared__ float4 lds_tile[];
@@ -213,9 +218,6 @@ void sddmm_tile_kernel(const TileArgs a)
         asm("" : "+v"(base_step[t]));  // one register, not an expression to be re-associated with each use
     }
 
-    // this launch covers K elements [k_off, k_off + 4*K4) of rows that are row_k4 float4 long
-    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (a.k_off >> 2);
-    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (a.k_off >> 2);
     const int row_k4 = a.K >> 2;
 
     // This workgroup's share of the stream: either the items b, b + grid, ... of an item
@@ -237,6 +239,14 @@ void sddmm_tile_kernel(const TileArgs a)
         n_steps = 0;
         for (int u = unit; u < a.n_units && a.unit_ptr[u] < hi; ++u) ++n_steps;
     }
+    const int n_slices = FUSED ? a.n_slices : 1;
+    for (int sl = 0; sl < n_slices; ++sl) {
+    const bool first_slice = sl == 0, last_slice = sl + 1 == n_slices;  // (used by the FUSED form only)
+    // this pass covers K elements [k_off, k_off + 4*K4) of rows that are row_k4 float4 long
+    const int k_off = a.k_off + sl * 4 * K4;
+    const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (k_off >> 2);
+    const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (k_off >> 2);
+    if (FUSED && sl > 0) __syncthreads();  // everyone is done with the slice before: its tile, and its partial results are stored
     int cur_tile = -1;
     for (int step = 0; step < n_steps; ++step) {
         int begin, end, tile;
@@ -346,7 +356,15 @@ void sddmm_tile_kernel(const TileArgs a)
         // ACC (K slices after the first): the previous slices' partial result, requested
         // one batch ahead of its use, from the position's own slot of a.part
         char *part_b = reinterpret_cast<char *>(a.part + begin);
-        auto issue_old = [&](Meta &m) { m.old = ACC ? *reinterpret_cast<const float *>(part_b + m.o) : 0.f; };
+        // (FUSED: the slot is read in every slice and ignored in the first: no load behind a branch)
+        auto issue_old = [&](Meta &m) {
+            if constexpr (FUSED) {
+                const float o = *reinterpret_cast<const float *>(part_b + m.o);
+                m.old = first_slice ? 0.f : o;
+            } else {
+                m.old = ACC ? *reinterpret_cast<const float *>(part_b + m.o) : 0.f;
+            }
+        };
         // wrow: float4 index of the row's first element in W
         auto issue_w = [&](float4 (&w)[KPL], uint32_t wrow) {
             const float4 *wbase[NB];  // piece j is at wbase[j % NB] + a compile-time offset
@@ -358,7 +376,7 @@ void sddmm_tile_kernel(const TileArgs a)
         };
         float pend_v;  // result of the batch before, not yet stored
         uint32_t pend_p, pend_o;
-        const bool to_part = PART && a.to_part != 0;  // (uniform)
+        const bool to_part = PART && (FUSED ? !last_slice : a.to_part != 0);  // (uniform)
         // (gather form: a position whose index carries bit 31 is padding that worked on
         // another row's column; its result goes to a scratch line instead of the output)
         // (one store whose address is selected, not a branch around two stores: a branch inside the
@@ -415,8 +433,8 @@ void sddmm_tile_kernel(const TileArgs a)
             // would sit, unfinished, in front of the loads that batch waits for.  In a
             // whole batch it needs no predicate: a padding position repeats a nonzero of
             // its own group and so writes that nonzero's own result a second time.
-            if constexpr (RESIDUAL) pend_v = ACC ? m.old - acc[0] : v - acc[0];
-            else pend_v = ACC ? fmaf(acc[0], v, m.old) : acc[0] * v;
+            if constexpr (RESIDUAL) pend_v = ACC ? m.old - acc[0] : FUSED ? (first_slice ? v : m.old) - acc[0] : v - acc[0];
+            else pend_v = (ACC || FUSED) ? fmaf(acc[0], v, m.old) : acc[0] * v;
             pend_p = m.p;
             pend_o = m.o;
         };
@@ -479,6 +497,16 @@ void sddmm_tile_kernel(const TileArgs a)
             if (begin + (bf << 6) + lane < end) flush();
         }
     }
+    }
+}
+
+// The all-slices-in-one-launch form exists for slices of 128 elements on groups of 8 lanes only (what the
+// planner uses for K > 128); null for the other variants.
+template <int G, int KPL, int VMODE, int NW, bool GATHER>
+TileFn fused_slices_kernel()
+{
+    if constexpr (G == 8 && KPL == 4) return (TileFn)sddmm_tile_kernel<G, KPL, VMODE, NW, GATHER, 3>;
+    else return nullptr;
 }
 
 }  // namespace

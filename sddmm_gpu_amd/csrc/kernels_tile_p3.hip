@@ -8,7 +8,8 @@ namespace sddmm {
 TileFn tile_kernel_part3(const TileVariant &v, int vmode, bool gather, int slice, int nwaves)
 {
 #define SDDMM_PICK_SLICE(g, kpl, vm, nw, ga)                                                                 \
-    (slice == 2 ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, ga, 2>                          \
+    (slice == 3 ? fused_slices_kernel<g, kpl, vm, nw, ga>()                                                 \
+     : slice == 2 ? (TileFn)sddmm_tile_kernel<g, kpl, (vm == 4 ? 3 : vm), nw, ga, 2>                        \
      : slice == 1 ? (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, ga, 1>                                        \
                   : (TileFn)sddmm_tile_kernel<g, kpl, vm, nw, ga, 0>)
 #define SDDMM_PICK(g, kpl, vm)                                                                              \

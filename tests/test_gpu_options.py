@@ -190,6 +190,36 @@ def test_banded_rows_walked_by_groups_of_workgroups(oracle, tmp_path, K):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("K,epilogue", [(256, "scale"), (512, "scale"), (384, "residual")])
+def test_k_slices_inside_one_launch_or_one_launch_each(oracle, K, epilogue):
+    """A sliced plan runs its K slices inside one kernel launch (fuse_slices = 1, what small matrices get) or one launch
+    per slice; the arithmetic per position is the same, so the results agree bit for bit, in every value mode."""
+    d = synth.make(3, 0.04, K=K, seed=11)
+    dev = torch.device(DEV)
+    W = d["W"].to(dev); H = d["H"].to(dev); dv = d["val"].to(dev)
+    outs = {}
+    for fuse in (0, 1):
+        plan = host_plan(d, K, split_min_nnz=0, dense_blocks=0, fuse_slices=fuse)
+        info = plan.info()
+        assert info["k_slice"] == 128 and info["n_launches"] == (2 if fuse else 2 * K // 128), info
+        res = []
+        for val in (0, dv.data_ptr()):   # the plan's stream-order values / the caller's sorted values
+            out = torch.full((d["nnz"],), float("nan"), device=dev)
+            if epilogue == "scale":
+                plan.execute(val, W.data_ptr(), H.data_ptr(), out.data_ptr())
+            else:
+                plan.execute_epilogue(val, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
+            torch.cuda.synchronize()
+            res.append(out.cpu())
+        assert torch.equal(res[0], res[1])
+        outs[fuse] = res[0]
+    assert torch.equal(outs[0], outs[1])
+    if epilogue == "scale":
+        check(d, outs[1].numpy(), oracle, K)
+    else:
+        residual_ok(outs[1].numpy(), d, oracle, K)
+
+
 def test_concurrent_executes_on_one_plan_and_concurrent_plan_creation(oracle):
     """The header's promise: a plan is immutable, sddmm_execute may be called from several threads on the same plan
     (each on its own stream, outputs apart); plans may also be built concurrently."""
