@@ -20,7 +20,7 @@ namespace {
 // again, merges the records of each cut row (at most two per chunk: the row that began before the chunk
 // and the row that ends after it) and scales the stored pieces.  Both kernels read the number of entries
 // from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.
-constexpr int kSmChunk = 4096;
+constexpr int kSmChunk = 4096;  // (recommender / R-MAT, chunk + merge kernel in us: 2048 -> 367 + 196 / 767 + 357; 4096 -> 289 + 133 / 626 + 218; 8192 -> 371 + 124 / 889 + 171)
 constexpr int kSmBlock = 256;
 constexpr int kSmRowsMax = kSmChunk + 128;  // row pointers of a chunk kept in LDS at a time
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
