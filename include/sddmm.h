@@ -85,6 +85,8 @@ typedef struct sddmm_plan_info {
     double plan_ms;       /* host time spent in the tiling pass + upload (a loaded plan: in reading the file) */
     int64_t dense_nnz;    /* nonzeros handled by the DENSE_BLOCK launch */
     int64_t dense_blocks; /* its 128 x 128 blocks */
+    int64_t matrix_nnz;   /* nonzeros of the LDS_TILE launch computed by its matrix-core waves (counted in class_nnz[0]) */
+    int64_t matrix_rows;  /* the rows they belong to */
 } sddmm_plan_info;
 
 const char *sddmm_last_error(void);
@@ -242,6 +244,13 @@ typedef struct sddmm_plan_options {
     int32_t dense_rb_group;     /* row blocks swept together by one die             [SDDMM_DENSE_RB_GROUP] */
     int32_t fuse_slices;        /* 0/1 the K slices of a launch run inside one kernel
                                    launch (-1: where the stream is small)           [SDDMM_FUSE_SLICES]   */
+    int32_t matrix_rows;        /* 1: the heaviest rows of an LDS_TILE launch go, as 32 x 32
+                                   blocks, to matrix-core waves inside the same workgroups
+                                   (0 and -1: off: fp32 MFMA and vector work of one SIMD do
+                                   not overlap, so the share measured slower)         [SDDMM_MATRIX_ROWS]   */
+    int32_t matrix_permille;    /* least fill of such a row, in 1/1000 of n_cols      [SDDMM_MATRIX_PERMILLE] */
+    int32_t matrix_waves;       /* matrix-core waves per workgroup: 4 (next to 12
+                                   vector waves) or 8 (next to 8)                     [SDDMM_MATRIX_WAVES]  */
     int32_t ignore_env;         /* 1: the environment is not consulted                                      */
     int64_t gather_slab_cols;   /* padded gather streams S in slabs of this many columns [SDDMM_GATHER_SLAB_COLS] */
     int64_t gather_panel_rows;  /* ... and, inside, in panels of this many listed rows   [SDDMM_GATHER_PANEL_ROWS] */

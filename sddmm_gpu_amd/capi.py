@@ -33,7 +33,8 @@ class PlanInfo(C.Structure):
                 ("lanes_per_nnz", c_int32), ("lds_bytes", c_int32), ("grid", c_int32), ("block", c_int32),
                 ("n_blocks", c_int64), ("device_bytes", c_int64), ("class_nnz", c_int64 * 3), ("class_rows", c_int64 * 3), ("padded_positions", c_int64),
                 ("short_batches", c_int64),
-                ("plan_ms", c_double), ("dense_nnz", c_int64), ("dense_blocks", c_int64)]
+                ("plan_ms", c_double), ("dense_nnz", c_int64), ("dense_blocks", c_int64), ("matrix_nnz", c_int64),
+                ("matrix_rows", c_int64)]
 
     def as_dict(self):
         return {f: (list(getattr(self, f)) if f.startswith("class_") else getattr(self, f)) for f, _ in self._fields_}
@@ -44,7 +45,7 @@ class PlanOptions(C.Structure):
     _fields_ = [(n, c_int32) for n in (
         "kernel", "tile_size_x", "tile_size_y", "k_slice", "tile_lanes", "tile_waves", "tile_assign", "tile_few_blocks",
         "tile_short_batches", "tile_deal", "tile_runs", "gather_lanes", "gather_padded", "gather_sink", "row_padded",
-        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "fuse_slices", "ignore_env")] + [(n, c_int64) for n in (
+        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "fuse_slices", "matrix_rows", "matrix_permille", "matrix_waves", "ignore_env")] + [(n, c_int64) for n in (
         "gather_slab_cols", "gather_panel_rows", "dense_min_nnz", "panel_bytes", "short_row_max", "stage_factor", "split_min_nnz")]
 
     @classmethod

@@ -55,6 +55,7 @@ struct Launch {
     // what the function pointers above were looked up with (they are looked up again when a saved plan is loaded)
     int32_t fn_kind = 0;  // 1 stream kernel (row gather), 2 stream kernel with an LDS tile, 3 tile kernel, 4 panel, 5 dense
     int32_t fn_g = 0, fn_kpl = 0, fn_exact = 0, fn_gather = 0, fn_nwaves = 0;
+    int32_t fn_nwm = 0;  // tile kernel: waves per workgroup that run the launch's matrix-core share (0: none)
     int32_t fused_slices = 0;  // sliced tile launch small enough that its K slices run inside one kernel launch
 };
 
@@ -198,6 +199,7 @@ void default_options(sddmm_plan_options &o)
     o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.fuse_slices = -1; o.gather_lanes = -1; o.gather_padded = -1;
     o.gather_sink = -1; o.row_padded = -1; o.unpadded_tile = -1; o.dense_blocks = -1; o.dense_permille = -1;
     o.dense_rb_group = -1; o.ignore_env = 0;
+    o.matrix_rows = -1; o.matrix_permille = -1; o.matrix_waves = -1;
     o.gather_slab_cols = -1; o.gather_panel_rows = -1; o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
 }
 
@@ -214,6 +216,7 @@ void apply_env_overrides(sddmm_plan_options &o)
     i32("SDDMM_GATHER_G", o.gather_lanes); i32("SDDMM_GATHER_PADDED", o.gather_padded); i32("SDDMM_GATHER_SINK", o.gather_sink);
     i32("SDDMM_ROW_PADDED", o.row_padded); i32("SDDMM_UNPADDED_TILE", o.unpadded_tile); i32("SDDMM_DENSE", o.dense_blocks);
     i32("SDDMM_DENSE_PERMILLE", o.dense_permille); i32("SDDMM_DENSE_RB_GROUP", o.dense_rb_group);
+    i32("SDDMM_MATRIX_ROWS", o.matrix_rows); i32("SDDMM_MATRIX_PERMILLE", o.matrix_permille); i32("SDDMM_MATRIX_WAVES", o.matrix_waves);
     i64("SDDMM_GATHER_SLAB_COLS", o.gather_slab_cols); i64("SDDMM_GATHER_PANEL_ROWS", o.gather_panel_rows); i64("SDDMM_DENSE_MIN_NNZ", o.dense_min_nnz); i64("SDDMM_PANEL_BYTES", o.panel_bytes);
     i64("SDDMM_SHORT_ROW_MAX", o.short_row_max); i64("SDDMM_STAGE_FACTOR", o.stage_factor);
     i64("SDDMM_SPLIT_MIN_NNZ", o.split_min_nnz);
@@ -235,6 +238,16 @@ int resolve_functions(Launch &L)
     }
     case 3: {
         const TileVariant tv{L.fn_g, L.fn_kpl};
+        if (L.fn_nwm > 0) {  // (a launch with a matrix-core share covers all of K: one form per value mode)
+            for (int vm = 0; vm < 5; ++vm) {
+                L.tfns[vm][0] = tile_kernel_mf(vm, L.fn_nwaves, L.fn_nwm);
+                if (!L.tfns[vm][0]) return fail(SDDMM_ERR_ARG, "plan: no tile kernel with %d + %d waves", L.fn_nwaves, L.fn_nwm);
+                HIP_TRY(hipFuncSetAttribute((const void *)L.tfns[vm][0], hipFuncAttributeMaxDynamicSharedMemorySize, L.lds));
+            }
+            L.fused_slices = 0;
+            L.tfn = L.tfns[0][0];
+            return SDDMM_OK;
+        }
         for (int vm = 0; vm < 5; ++vm)
             for (int ac = 0; ac < 4; ++ac) {
                 L.tfns[vm][ac] = tile_kernel(tv, vm, L.fn_gather != 0, ac, L.fn_nwaves);
@@ -473,7 +486,7 @@ constexpr size_t kStreamSlack = 256;  // readable entries behind a tile stream's
 
 // Tile launch: the rows' nonzeros in tile order (tiles of x columns), every
 // (row, tile) run padded to a multiple of G stream positions.
-int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_rows, int want_g, int ks,
+int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t panel_rows, int want_g, int ks,
              sddmm_plan_info *I, bool gather = false, bool x_explicit = false)
 {
     // gather: the padded stream in plain row order (one tile as wide as S, one panel),
@@ -487,7 +500,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         if (c.opt.gather_slab_cols > 0) x = (int32_t)std::min<int64_t>(x, c.opt.gather_slab_cols);
         panel_rows = c.opt.gather_panel_rows > 0 ? (int32_t)std::min<int64_t>(c.opt.gather_panel_rows, INT32_MAX) : INT32_MAX;
     }
-    L.rows = (int64_t)rows.size();
+    L.rows = (int64_t)rows_in.size();
     const TileVariant tv = pick_tile_variant(ks, want_g);  // ks: K elements per launch (K itself or a slice of it)
     // 12 waves per workgroup measured 2-5 % faster than 16 on slices of 64 and 128, slower on 32
     int nwaves = gather ? 4 : (int)(c.opt.tile_waves > 0 ? c.opt.tile_waves : (ks >= 64 ? 12 : 16));
@@ -495,11 +508,11 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
     if (!tv.G || !tile_kernel(tv, 0, gather, 0, nwaves)) return fail(SDDMM_ERR_ARG, "plan: no tile kernel for K = %d", c.K);
     L.fn_kind = 3; L.fn_g = tv.G; L.fn_kpl = tv.KPL; L.fn_gather = gather; L.fn_nwaves = nwaves;
     const int G = tv.G;
-    L.nnz = list_nnz(c, rows);
+    L.nnz = list_nnz(c, rows_in);
     if (L.nnz == 0) return SDDMM_OK;
     // the kernel addresses W (and, in the gather form, H) rows by 32-bit float4 indices
     if ((int64_t)c.n_rows * (c.K / 4) > (int64_t)UINT32_MAX || (gather && (int64_t)c.n_cols * (c.K / 4) > (int64_t)UINT32_MAX))
-        return add_row_gather(c, rows, false);
+        return add_row_gather(c, rows_in, false);
     // Work assignment.  grid2d: every workgroup owns one column tile for good (its H
     // tile is staged once) and one of `shares` row blocks that are the same for all
     // tiles, so the workgroups of different tiles read the same W rows at about the same
@@ -538,6 +551,52 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         }
         if (grid2d) panel_rows = INT32_MAX;
     }
+    // Matrix-core share (only on request, matrix_rows = 1).  Rows filled to a good part of n_cols leave the
+    // stream and are computed as whole 32 x 32 blocks (32 such rows x 32 consecutive columns) by extra
+    // waves of the same workgroups (see TileArgs::mf_*).  Whole multiples of 256 rows, so that every die
+    // gets the same number of groups of 32.  Measured on the recommender shape at K = 128 it loses: a
+    // v_mfma_f32 occupies its SIMD's vector unit for as long as it runs (SQ_VALU_MFMA_COEXEC_CYCLES
+    // reads 0 with both kinds of waves resident), so the two kinds of work add up instead of overlapping
+    // (vector waves alone 0.38 ms, the MFMA stream alone 0.21 ms, together 0.62 ms; the stream with
+    // every row 0.63 ms), and what the matrix cores save per flop goes to the cells of a block that hold
+    // no nonzero.
+    std::vector<int32_t> mf_rows, rest_rows;
+    int mf_nwm = 0;
+    int64_t mf_nnz = 0;
+    if (xcd_local && !gather && tv.G == 8 && tv.KPL == 4 && ks == c.K && (nwaves == 12 || c.opt.tile_waves == 8) && !c.orig &&
+        c.opt.matrix_rows > 0 &&
+        c.cus % 8 == 0 && c.n_cols >= 32) {
+        const int nwm = c.opt.matrix_waves == 8 ? 8 : 4;
+        const int nwv = nwm == 8 || c.opt.tile_waves == 8 ? 8 : 12;
+        const int64_t lds_need = (int64_t)x * ks * 4 + kMfLdsExtra + (int64_t)nwm * kMfLdsPerWave;
+        const int64_t permille = c.opt.matrix_permille > 0 ? c.opt.matrix_permille : 250;
+        const int64_t min_deg = std::max<int64_t>(32, permille * c.n_cols / 1000);
+        const int64_t n_cb = (c.n_cols + 31) / 32;
+        std::vector<int32_t> heavy;
+        for (int32_t r : rows_in)
+            if (c.row_ptr[r + 1] - c.row_ptr[r] >= min_deg) heavy.push_back(r);
+        std::stable_sort(heavy.begin(), heavy.end(), [&](int32_t u, int32_t v) {
+            return c.row_ptr[u + 1] - c.row_ptr[u] > c.row_ptr[v + 1] - c.row_ptr[v];
+        });
+        heavy.resize(heavy.size() / 256 * 256);  // (the lightest of them stay in the stream)
+        const int64_t n_groups = (int64_t)heavy.size() / 32;
+        const int64_t h_nnz = list_nnz(c, heavy);
+        const bool fits = lds_need <= kLdsMaxBytes && tile_kernel_mf(0, nwv, nwm) != nullptr &&
+                          n_groups * n_cb * 256 < ((int64_t)1 << 31) && n_cb < (1 << 17) && n_groups < (1 << 17);
+        if (fits && !heavy.empty() && heavy.size() < rows_in.size()) {
+            std::vector<uint8_t> is_heavy((size_t)c.n_rows, 0);
+            for (int32_t r : heavy) is_heavy[(size_t)r] = 1;
+            for (int32_t r : rows_in)
+                if (!is_heavy[(size_t)r]) rest_rows.push_back(r);
+            mf_rows.swap(heavy);
+            mf_nwm = nwm;
+            mf_nnz = h_nnz;
+            nwaves = nwv;
+            L.fn_nwaves = nwaves;
+        }
+    }
+    const std::vector<int32_t> &rows = mf_nwm ? rest_rows : rows_in;
+    const int64_t stream_nnz = L.nnz - mf_nnz;
     // panel_local (decided below, once the tiling is known): a matrix with more column tiles than
     // workgroups whose rows touch only a few tiles each (banded shapes) is cut into a few row ranges,
     // and each range is walked from top to bottom by a group of workgroups of one die that hold the
@@ -584,7 +643,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
             int64_t acc = 0; int sidx = 1;
             for (size_t i = 0; i < rows.size() && sidx < n_shares; ++i) {
                 acc += c.row_ptr[rows[i] + 1] - c.row_ptr[rows[i]];
-                while (sidx < n_shares && acc >= L.nnz * sidx / n_shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
+                while (sidx < n_shares && acc >= stream_nnz * sidx / n_shares) cut[sidx++] = (i + 1 < rows.size()) ? rows[i + 1] : INT32_MAX;
             }
         };
         make_cuts(shares);
@@ -971,6 +1030,48 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         if (int rc = c.up(&d_sink, std::vector<float>(256 * 64, 0.f))) return rc;
         a.sink = d_sink;
     }
+    if (mf_nwm) {
+        // Groups of 32 rows in order of length; group k of that order belongs to die k % 8 and is stored as
+        // group (k % 8) * Gd + k / 8, so that a die's groups are consecutive.
+        const int64_t n_cb = (c.n_cols + 31) / 32;
+        const int64_t NG = (int64_t)mf_rows.size() / 32, Gd = NG / 8;
+        std::vector<int32_t> slot_rows((size_t)NG * 32);
+        for (int64_t k = 0; k < NG; ++k)
+            std::copy(mf_rows.begin() + k * 32, mf_rows.begin() + (k + 1) * 32, slot_rows.begin() + ((k % 8) * Gd + k / 8) * 32);
+        std::vector<uint2> rowinfo((size_t)(NG * n_cb * 32), make_uint2(0u, 0u));
+        parallel_ranges(NG, 1, [&](int64_t gb, int64_t ge, int) {
+            for (int64_t g = gb; g < ge; ++g) {
+                const int64_t die = g / Gd, k = g - die * Gd;
+                uint2 *base = rowinfo.data() + (size_t)(die * Gd * n_cb) * 32;
+                for (int i = 0; i < 32; ++i) {
+                    const int32_t r = slot_rows[(size_t)g * 32 + i];
+                    for (int32_t p = c.row_ptr[r]; p < c.row_ptr[r + 1]; ++p) {
+                        const int32_t col = c.col_ind[p];
+                        uint2 &e = base[((size_t)(col >> 5) * Gd + k) * 32 + i];
+                        if (!e.x) e.y = (uint32_t)p;
+                        e.x |= 1u << (col & 31);
+                    }
+                }
+            }
+        });
+        uint2 *d_ri = nullptr;
+        int32_t *d_rows = nullptr;
+        if (int rc = c.up(&d_ri, rowinfo)) return rc;
+        if (int rc = c.up(&d_rows, slot_rows)) return rc;
+        float4 *d_hp = nullptr, *d_wp = nullptr;
+        const size_t hp_bytes = (size_t)n_cb << 14, wp_bytes = (size_t)NG << 14;
+        HIP_TRY(hipMalloc((void **)&d_hp, hp_bytes));
+        c.P->owned.push_back({d_hp, hp_bytes, true});
+        HIP_TRY(hipMalloc((void **)&d_wp, wp_bytes));
+        c.P->owned.push_back({d_wp, wp_bytes, true});
+        c.dev_bytes += (int64_t)(hp_bytes + wp_bytes);
+        a.mf_hp = d_hp; a.mf_wp = d_wp; a.mf_rowinfo = d_ri; a.mf_rows = d_rows;
+        a.mf_groups = (int32_t)NG; a.mf_n_cb = (int32_t)n_cb;
+        a.tile_bytes = (int32_t)((int64_t)x * ks * 4);
+        L.fn_nwm = mf_nwm;
+        c.P->info.matrix_nnz += mf_nnz;
+        c.P->info.matrix_rows += (int64_t)mf_rows.size();
+    }
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     if (grid2d) {
         WorkItem *d_items = nullptr;
@@ -978,8 +1079,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows, int32_t x, int32_t panel_
         a.items = d_items; a.n_items = (int32_t)items.size();
         L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)items.size()));
     }
-    L.block = nwaves * 64;
+    L.block = (nwaves + mf_nwm) * 64;
     L.lds = gather ? 0 : (int32_t)((int64_t)x * ks * 4);
+    if (mf_nwm) {
+        L.lds += kMfLdsExtra + mf_nwm * kMfLdsPerWave;
+        // (every workgroup's matrix-core waves take a share of their die's pairs: all workgroups must exist)
+        if (L.grid != c.cus) return fail(SDDMM_ERR_ARG, "plan: matrix-core share on a launch of %d workgroups", L.grid);
+    }
     L.k_slice = ks;
     if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
     if (int rc = resolve_functions(L)) return rc;
@@ -1515,6 +1621,11 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.val = val;
         ta.sval = d_val ? nullptr : L.sval;
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
+        ta.nnz = (int32_t)I.nnz;
+        if (ta.mf_groups > 0) {  // the matrix-core share reads its operands from packed copies of H and of its W rows
+            ta.k_off = 0;
+            launch_mf_pack(ta, stream);
+        }
         const int vm = residual ? (ta.sval ? 3 : 4) : ta.sval ? 0 : (val ? 1 : 2);
         const bool sliced = L.k_slice < I.K;
         if (sliced && L.fused_slices) {
@@ -1621,7 +1732,7 @@ void launch_pointer_fields(Launch &L, std::vector<void *> &fields)
 {
     fields = {&L.ka.perm, &L.ka.scol, &L.ka.seg_row, &L.ka.batch_seg, &L.ka.batch_mask, &L.ka.items,
             &L.ta.perm, &L.ta.scol, &L.ta.grow, &L.ta.scol16, &L.ta.pbase, &L.ta.btype, &L.ta.part, &L.ta.sink, &L.ta.unit_ptr,
-            &L.ta.unit_tile, &L.ta.items,
+            &L.ta.unit_tile, &L.ta.items, &L.ta.mf_hp, &L.ta.mf_wp, &L.ta.mf_rowinfo, &L.ta.mf_rows,
             &L.pa.slot_row, &L.pa.panel_tiles,
             &L.da.slot_rows, &L.da.slot_cols, &L.da.slot_range, &L.da.nz_p, &L.da.nz_rc,
             &L.sval, &L.perm};
@@ -1661,6 +1772,7 @@ bool same_options(const sddmm_plan_options &a, const sddmm_plan_options &b)
            a.gather_lanes == b.gather_lanes && a.gather_padded == b.gather_padded && a.gather_sink == b.gather_sink &&
            a.row_padded == b.row_padded && a.unpadded_tile == b.unpadded_tile && a.dense_blocks == b.dense_blocks &&
            a.dense_permille == b.dense_permille && a.dense_rb_group == b.dense_rb_group &&
+           a.matrix_rows == b.matrix_rows && a.matrix_permille == b.matrix_permille && a.matrix_waves == b.matrix_waves &&
            a.gather_slab_cols == b.gather_slab_cols && a.gather_panel_rows == b.gather_panel_rows &&
            a.dense_min_nnz == b.dense_min_nnz && a.panel_bytes == b.panel_bytes && a.short_row_max == b.short_row_max &&
            a.stage_factor == b.stage_factor && a.split_min_nnz == b.split_min_nnz;

@@ -85,6 +85,23 @@ struct TileArgs {
     int32_t K;           // row length of W and H
     int32_t k_off;       // first K element covered by this launch (the kernel's own width is 4*G*KPL)
     int32_t n_slices;    // the all-slices-in-one-launch form: K slices walked inside the launch, from k_off on
+    // Matrix-core share of a launch (kernel variants with NWM > 0; mf_groups == 0: none).  The heaviest
+    // rows, in groups of 32, are multiplied as whole 32 x 32 blocks against blocks of 32 consecutive
+    // columns by the last NWM waves of every workgroup, from operands packed by mf_pack_kernel:
+    //   mf_hp[(cb * 32 + p) * 32 + j] = float4 p of the K slice of H row 32 cb + j (zero beyond n_cols)
+    //   mf_wp[(g * 32 + p) * 32 + i]  = float4 p of the K slice of W row mf_rows[32 g + i]
+    // (an MFMA operand load of one wave is then 1 KB of consecutive addresses).  Groups [die * G, (die + 1) * G),
+    // G = mf_groups / 8, belong to the workgroups of that die (workgroup b runs on die b % 8); a die's
+    // (group, column block) pairs are numbered column block by column block, q = cb * G + (g - die * G), and
+    // mf_rowinfo[(die * G * mf_n_cb + q) * 32 + i] = {bit j set: S has (row i of the group, column 32 cb + j);
+    // sorted position of the row's first nonzero in that block}: the nonzero of bit j sits at that
+    // position plus the number of set bits below j.
+    const float4 *mf_hp, *mf_wp;
+    const uint2 *mf_rowinfo;
+    const int32_t *mf_rows;   // [32 * mf_groups] rows of the groups (a short last group repeats a row, with empty masks)
+    int32_t mf_groups, mf_n_cb;
+    int32_t nnz;              // of S (bound for value reads)
+    int32_t tile_bytes;       // bytes of the H tile in LDS (the matrix-core waves' own LDS follows it)
 };
 struct TileVariant {
     int G, KPL;  // lanes per nonzero, float4 per lane; K == 4*G*KPL
@@ -101,6 +118,13 @@ TileVariant pick_tile_variant(int K, int want_g);
 // gather: H rows from global memory, 4 waves per workgroup (otherwise H tiles in LDS, nwaves = 16 or 12 waves)
 // slice: 0 the launch covers all of K, 1 first of several K slices, 2 a later one (see the kernel template)
 TileFn tile_kernel(const TileVariant &v, int vmode, bool gather, int slice, int nwaves);
+// The variant with a matrix-core share (TileArgs::mf_*): groups of 8 lanes on rows of 128 elements, all of K
+// in one launch, nw vector waves + nwm matrix-core waves per workgroup ((12, 4), (8, 8) or (8, 4)).
+TileFn tile_kernel_mf(int vmode, int nw, int nwm);
+constexpr int kMfLdsExtra = 64;        // bytes of LDS behind the H tile for the vector waves' barrier counter ...
+constexpr int kMfLdsPerWave = 512;     // ... and for each matrix-core wave's row masks
+// packs the operands of the matrix-core share (a.mf_hp from a.H, a.mf_wp from a.W through a.mf_rows) on `stream`
+void launch_mf_pack(const TileArgs &a, void *stream);
 
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);

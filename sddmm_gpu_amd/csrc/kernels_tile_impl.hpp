@@ -33,6 +33,19 @@ using namespace sddmm;
 
 namespace {
 
+// Stream data (positions, LDS offsets, values, W row numbers) is read once per launch: with the
+// non-temporal hint it does not displace the W rows and output lines that the caches are needed
+// for.  Same-box A/B: the LDS-tile form covering K = 128 in one launch, recommender shape: tile
+// kernel 0.638 -> 0.617 ms; the compact stream of K = 32: 0.354 -> 0.384 ms; K slices: no change
+// (recommender, K = 256) or + 2 % (banded, K = 512); the gather form + 2 %; on the stores + 12 %
+// (the pieces of an output line come from different tiles and have to meet in L2).  So the hint
+// is given by the uncompacted single-launch LDS-tile form only.
+template <bool STREAMING, class T> __device__ __forceinline__ T ld_meta(const T *p)
+{
+    if constexpr (STREAMING) return __builtin_nontemporal_load(p);
+    else return *p;
+}
+
 typedef float vec4f __attribute__((ext_vector_type(4)));  // a plain vector: loadable through an LDS-qualified pointer
 
 __device__ __forceinline__ float dot4(const float4 &a, const float4 &b, float acc)
@@ -148,6 +161,122 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
     }
 }
 
+// The matrix-core share of a tile launch, run by the last NWM waves of every workgroup while the
+// other waves walk the stream (see TileArgs).  A wave keeps the B operand of one column block
+// (32 columns x 128 elements of H: 64 registers) and streams the A operands of its die's row
+// groups past it: 64 v_mfma_f32_32x32x2_f32 per (group, block) pair, plain fp32 in and out.  The
+// results leave the accumulators directly: accumulator register v of lane l is the dot product of
+// row 8 (v / 4) + 4 (l / 32) + v % 4 of the group and column l % 32 of the block; where the row's
+// mask has that column's bit, it goes to the row's base position plus the number of set bits below
+// the column (a row's nonzeros inside 32 consecutive columns are consecutive in the sorted S).
+// ri_slot: 512 bytes of LDS of this wave's own.
+// AHEAD: A operands requested ahead of the one in use; CHUNK: results stored per round of value
+// loads (both sized by the registers a wave has: 128 with 16 waves per workgroup, 170 with 12).
+template <int VMODE, int AHEAD, int CHUNK>
+__device__ __forceinline__ void matrix_core_waves(const TileArgs &a, int mw, int nmw, int lane, uint2 *ri_slot)
+{
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+    constexpr bool RESIDUAL = VMODE >= 3;
+    constexpr bool HASVAL = VMODE != 2;
+    const int die = blockIdx.x & 7;
+    const int G = a.mf_groups >> 3;
+    const int wpd = (int)(gridDim.x >> 3) * nmw;            // matrix-core waves per die
+    const int w = (int)(blockIdx.x >> 3) * nmw + mw;        // this wave's number among them
+    const int64_t P = (int64_t)G * a.mf_n_cb;               // pairs of the die
+    int q = __builtin_amdgcn_readfirstlane((int)(P * w / wpd));
+    const int q1 = __builtin_amdgcn_readfirstlane((int)(P * (w + 1) / wpd));
+    if (q >= q1) return;
+    const int g0 = die * G;
+    int cb = __builtin_amdgcn_readfirstlane(q / G), gi = q - cb * G;
+    // Operands come through buffer loads: (descriptor in scalar registers) + (scalar byte offset of the
+    // pair and step) + (16 bytes per lane), so that no lane computes a 64-bit address.
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit elements
+    const __amdgpu_buffer_rsrc_t rs_h =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float4 *>(a.mf_hp), 0, a.mf_n_cb << 14, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_w =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float4 *>(a.mf_wp), 0, a.mf_groups << 14, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs_ri =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint2 *>(a.mf_rowinfo), 0, (a.mf_groups * a.mf_n_cb) << 8, kRsrcFlags);
+    const int ri0 = (g0 * a.mf_n_cb) << 8;
+    const int l16 = lane << 4, l8 = (lane & 31) << 3;
+    const uint32_t lane_bit = 1u << (lane & 31), lane_lt = lane_bit - 1u;
+    const int half4 = (lane >> 5) << 2;
+    const uint32_t last = (uint32_t)(a.nnz - 1);
+    vec4f b[16];
+    auto load_b = [&](int c) {
+#pragma unroll
+        for (int s = 0; s < 16; ++s)
+            b[s] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(rs_h, l16, (c << 14) + s * 1024, 0));
+    };
+    // row masks and base positions of a pair go through this wave's LDS slot; those of the next
+    // pair are requested while this one is computed
+    v2u rin = __builtin_amdgcn_raw_buffer_load_b64(rs_ri, l8, ri0 + (q << 8), 0);
+    load_b(cb);
+    ri_slot[lane] = make_uint2(rin.x, rin.y);
+    while (true) {
+        const int a_off = (g0 + gi) << 14;
+        constexpr int kAhead = AHEAD;
+        vec4f aw[kAhead];
+#pragma unroll
+        for (int s = 0; s < kAhead; ++s)
+            aw[s] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(rs_w, l16, a_off + s * 1024, 0));
+        __builtin_amdgcn_sched_barrier(0);
+        v16f acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[s % kAhead].x, b[s].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[s % kAhead].y, b[s].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[s % kAhead].z, b[s].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[s % kAhead].w, b[s].w, acc, 0, 0, 0);
+            if (s + kAhead < 16) {
+                aw[s % kAhead] = __builtin_bit_cast(vec4f, __builtin_amdgcn_raw_buffer_load_b128(rs_w, l16, a_off + (s + kAhead) * 1024, 0));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // the next pair's masks and positions arrive while this pair's results are stored
+        const int qn = min(q + 1, q1 - 1);
+        rin = __builtin_amdgcn_raw_buffer_load_b64(rs_ri, l8, ri0 + (qn << 8), 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // (the slot was written by this wave: LDS operations of one wave complete in order)
+        __builtin_amdgcn_wave_barrier();
+        constexpr int kChunk = CHUNK;
+#pragma unroll
+        for (int h = 0; h < 16 / kChunk; ++h) {
+            uint32_t idx[kChunk], has[kChunk];
+            float sv[kChunk];
+#pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const int v = kChunk * h + u;
+                const uint2 r = ri_slot[8 * (v >> 2) + (v & 3) + half4];
+                idx[u] = (uint32_t)__builtin_popcount(r.x & lane_lt) + r.y;
+                has[u] = r.x & lane_bit;
+            }
+            if constexpr (HASVAL) {
+#pragma unroll
+                for (int u = 0; u < kChunk; ++u) sv[u] = a.val[min(idx[u], last)];
+            }
+#pragma unroll
+            for (int u = 0; u < kChunk; ++u) {
+                const float d = acc[kChunk * h + u];
+                float o;
+                if constexpr (RESIDUAL) o = sv[u] - d;
+                else if constexpr (HASVAL) o = d * sv[u];
+                else o = d;
+                if (has[u]) a.out[idx[u]] = o;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // (the slot is written again only after these reads)
+        ri_slot[lane] = make_uint2(rin.x, rin.y);
+        if (++q >= q1) break;
+        if (++gi == G) {
+            gi = 0;
+            ++cb;
+            load_b(cb);
+        }
+    }
+}
+
 // VMODE: where S.val comes from -- 0: a.sval (stream order), 1: a.val (sorted
 // order, read through the position), 2: nowhere (no scaling); 3 and 4: as 0 and 1
 // with the residual epilogue, out = val - dot (K slices after the first: out -= dot,
@@ -166,8 +295,12 @@ __device__ __forceinline__ void transpose_reduce_step(float (&acc)[G], int l)
 // launch costs as much as its work): a wave meets the same positions in every slice, so the partial
 // results it left in a.part are its own, and a workgroup barrier between the slices is all the
 // ordering needed.
-template <int G, int KPL, int VMODE, int NW, bool GATHER, int SLICE>
-__global__ __launch_bounds__(NW * 64)
+// NWM > 0: the workgroup has NWM more waves, which run the matrix-core share of the launch
+// (matrix_core_waves) and take no part in staging or in the stream; the NW vector waves then
+// synchronise among themselves through a counter in LDS, since a hardware barrier would wait
+// for all waves.
+template <int G, int KPL, int VMODE, int NW, bool GATHER, int SLICE, int NWM = 0>
+__global__ __launch_bounds__((NW + NWM) * 64)
 void sddmm_tile_kernel(const TileArgs a)
 {
     constexpr bool FUSED = SLICE == 3;
@@ -180,6 +313,7 @@ void sddmm_tile_kernel(const TileArgs a)
     constexpr bool SORTED_VAL = VMODE == 1 || (VMODE == 4 && !ACC);  // values read through the position
     constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
     constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
+    constexpr bool STREAM_HINT = !GATHER && !COMPACT && SLICE == 0;  // (see ld_meta)
     constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
     // SHORTS: a batch may be marked "short" in a.btype: each of its groups then holds at most G/2
     // nonzeros in its first G/2 positions and the same ones again in the other G/2.  With the
@@ -197,6 +331,31 @@ void sddmm_tile_kernel(const TileArgs a)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: loop bounds stay in SGPRs
+    // barrier among the vector waves: every wave adds one to the counter and waits for the sum to
+    // reach NW times the number of barriers so far
+    uint32_t sync_target = 0;
+    uint32_t *sync_ctr = nullptr;
+    if constexpr (NWM > 0) {
+        char *extra = reinterpret_cast<char *>(lds_tile) + a.tile_bytes;
+        sync_ctr = reinterpret_cast<uint32_t *>(extra);
+        if (threadIdx.x == 0) *sync_ctr = 0;
+        __syncthreads();  // the only hardware barrier: all waves are still here
+        if (wave >= NW) {
+            if (a.mf_groups > 0)
+                matrix_core_waves<VMODE, (NW + NWM > 12 ? 6 : 8), (NW + NWM > 12 ? 4 : 16)>(a, wave - NW, NWM, lane, reinterpret_cast<uint2 *>(extra + 64) + (wave - NW) * 64);
+            return;
+        }
+    }
+    auto wg_sync = [&]() {
+        if constexpr (NWM == 0) {
+            __syncthreads();
+        } else {
+            sync_target += NW;
+            if (lane == 0) __hip_atomic_fetch_add(sync_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+            while (__hip_atomic_load(sync_ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < sync_target)
+                __builtin_amdgcn_s_sleep(1);
+        }
+    };
     const int l = lane & (G - 1);
     const int rot = (lane / G) & (NB - 1);
 
@@ -246,7 +405,7 @@ void sddmm_tile_kernel(const TileArgs a)
     const int k_off = a.k_off + sl * 4 * K4;
     const float4 *__restrict__ W4 = reinterpret_cast<const float4 *>(a.W) + (k_off >> 2);
     const float4 *__restrict__ H4 = reinterpret_cast<const float4 *>(a.H) + (k_off >> 2);
-    if (FUSED && sl > 0) __syncthreads();  // everyone is done with the slice before: its tile, and its partial results are stored
+    if (FUSED && sl > 0) wg_sync();  // everyone is done with the slice before: its tile, and its partial results are stored
     int cur_tile = -1;
     for (int step = 0; step < n_steps; ++step) {
         int begin, end, tile;
@@ -265,7 +424,7 @@ void sddmm_tile_kernel(const TileArgs a)
         }
         if (end <= begin) continue;
         if (!GATHER && tile != cur_tile) {
-            if (cur_tile >= 0) __syncthreads();  // everyone is done with the previous tile
+            if (cur_tile >= 0) wg_sync();  // everyone is done with the previous tile
             cur_tile = tile;
             const int tile_base = tile * a.tile_x;
             const int rows = min(a.tile_x, a.n_cols - tile_base);
@@ -289,7 +448,7 @@ void sddmm_tile_kernel(const TileArgs a)
                 const int r = i / K4, q = i - r * K4;
                 lds_tile[i] = src[(size_t)r * row_k4 + q];
             }
-            __syncthreads();
+            wg_sync();
         }
         const int nb = (end - begin + 63) >> 6;
         // (the division runs on the vector unit; the results are uniform and go back to scalar
@@ -319,16 +478,16 @@ void sddmm_tile_kernel(const TileArgs a)
         auto issue_meta = [&]() -> Meta {
             Meta m;
             if constexpr (COMPACT) {
-                const uint32_t g = *reinterpret_cast<const uint32_t *>(grow_b + og);
+                const uint32_t g = ld_meta<STREAM_HINT>(reinterpret_cast<const uint32_t *>(grow_b + og));
                 m.wrow = g & ~(uint32_t)(G - 1);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + og) + min((uint32_t)l, g & (uint32_t)(G - 1));
-                m.col = (int)*reinterpret_cast<const uint16_t *>(scol_b + (o4 >> 1)) << ROW_SHIFT;
+                m.p = ld_meta<STREAM_HINT>(reinterpret_cast<const uint32_t *>(perm_b + og)) + min((uint32_t)l, g & (uint32_t)(G - 1));
+                m.col = (int)ld_meta<STREAM_HINT>(reinterpret_cast<const uint16_t *>(scol_b + (o4 >> 1))) << ROW_SHIFT;
             } else {
-                m.wrow = *reinterpret_cast<const uint32_t *>(grow_b + og);
-                m.p = *reinterpret_cast<const uint32_t *>(perm_b + o4);
-                m.col = *reinterpret_cast<const int *>(scol_b + o4);
+                m.wrow = ld_meta<STREAM_HINT>(reinterpret_cast<const uint32_t *>(grow_b + og));
+                m.p = ld_meta<STREAM_HINT>(reinterpret_cast<const uint32_t *>(perm_b + o4));
+                m.col = ld_meta<STREAM_HINT>(reinterpret_cast<const int *>(scol_b + o4));
             }
-            m.sv = STREAM_VAL ? *reinterpret_cast<const float *>(sval_b + o4) : 1.0f;
+            m.sv = STREAM_VAL ? ld_meta<STREAM_HINT>(reinterpret_cast<const float *>(sval_b + o4)) : 1.0f;
             m.o = o4;
             o4 += 256;
             og += 256 / G;
