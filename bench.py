@@ -161,6 +161,7 @@ def main():
     ap.add_argument("--tile-x", type=int, default=0)
     ap.add_argument("--tile-y", type=int, default=0)
     ap.add_argument("--no-sweep", action="store_true", help="skip the K = 32, 128, 256, 512 report")
+    ap.add_argument("--no-others", action="store_true", help="skip the other benchmark shapes (other_configs)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true", help="skip the sampled comparison with the CPU oracle")
     ap.add_argument("--opt", action="append", default=[], metavar="FIELD=VALUE",
@@ -198,17 +199,18 @@ def main():
 
     d = synth.make(args.config, args.scale, device=dev, K=args.K)
     K0 = d["K"]
-    sigma = float(d["W"].std())
 
-    def set_rank(K):
+    def set_rank(K, d=d):
         if K != d["K"]:
             g = torch.Generator(device=dev); g.manual_seed(1000 + K)
-            d["W"] = torch.randn(d["n_rows"], K, generator=g, device=dev) * sigma
-            d["H"] = torch.randn(d["n_cols"], K, generator=g, device=dev) * sigma
+            s = float(d["W"].std())
+            d["W"] = d["H"] = None
+            d["W"] = torch.randn(d["n_rows"], K, generator=g, device=dev) * s
+            d["H"] = torch.randn(d["n_cols"], K, generator=g, device=dev) * s
             d["K"] = K
 
-    def measure(K, steps=None, warmup=None, spinup=None, keep_out=False, **more):
-        set_rank(K)
+    def measure(K, steps=None, warmup=None, spinup=None, keep_out=False, d=d, **more):
+        set_rank(K, d)
         steps = args.steps if steps is None else steps
         warmup = args.warmup if warmup is None else warmup
         spinup = args.spinup_ms if spinup is None else spinup
@@ -389,6 +391,46 @@ def main():
     if not args.no_cpu:
         set_rank(K0)
         line["cpu_baseline"] = cpu_baseline(d, K0)
+    if not args.no_sweep and not args.no_others and args.config == 3 and args.scale == 1.0 and not opt_fields:
+        # The other benchmark shapes, each generated on the device, planned, spun up and timed like the main
+        # one (the same steps and warm-up), with its own sample against the CPU oracle: the uniform plumbing
+        # case, bag-of-words with the tile width the benchmark list states and with the planner's own, the
+        # R-MAT graph, and the banded shape at both of its ranks.
+        main_args = (args.tile_x, args.tile_y)
+        others = []
+        for cfg, K, tx in ((1, 32, 0), (2, 256, 192), (2, 256, 0), (4, 64, 0), (5, 512, 0), (5, 1024, 0)):
+            d.clear()
+            torch.cuda.empty_cache()
+            t_gen = time.perf_counter()
+            if not others or others[-1]["config"] != cfg:
+                d2 = synth.make(cfg, 1.0, device=dev, K=K)
+            torch.cuda.synchronize()
+            t_gen = time.perf_counter() - t_gen
+            args.tile_x, args.tile_y = tx, 0
+            r = measure(K, keep_out=not args.no_parity, d=d2)
+            i2 = r["info"]
+            row = {"config": cfg, "workload": names[cfg], "n_rows": d2["n_rows"], "n_cols": d2["n_cols"], "nnz": d2["nnz"], "K": K,
+                   "tile_size_x_asked": tx, "tile_size_x": i2["tile_size_x"], "tile_size_y": i2["tile_size_y"], "k_slice": i2["k_slice"],
+                   "kernel": KERNEL_NAMES[i2["kernel"]], "kernel_launches_per_step": i2["n_launches"],
+                   "ms_per_step": round(r["ms_per_step"], 5), "kernel_ms": round(r["kernel_ms_mean"], 5),
+                   "gflops": round(r["gflops"], 1), "alg_bytes_per_step": r["alg_bytes"], "alg_gbps": round(r["alg_gbps"], 1),
+                   "hbm_frac": round(r["frac"], 4), "plan_ms": round(i2["plan_ms"], 1), "generate_s": round(t_gen, 2),
+                   "kernels": [{"kernel": KERNEL_NAMES[p["kernel"]], "nnz": p["nnz"], "stream_positions": p["stream_positions"],
+                                "launches": p["n_kernel_launches"], "ms": round(p["ms"], 5)} for p in r["prof"]]}
+            tp = traffic_profile_path(cfg, 1.0, K, args.kernel, tx, 0, {})
+            if tp:
+                from sddmm_gpu_amd import rocprof
+                row["traffic"] = rocprof.traffic_from_profile_text(tp)
+                row["traffic_source"] = os.path.relpath(tp, ROOT) if row["traffic"] is not None else None
+            if not args.no_parity:
+                row["parity"] = parity_block(d2, K, r.pop("out"), torch)
+            others.append(row)
+            del r
+            print("other-config", json.dumps(row), file=sys.stderr, flush=True)
+        args.tile_x, args.tile_y = main_args
+        del d2
+        torch.cuda.empty_cache()
+        line["other_configs"] = others
     line["config"]["executes"] = executes[0]
     line["config"]["argv"] = sys.argv[1:]
     if args.from_prof:

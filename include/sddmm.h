@@ -17,7 +17,8 @@
  * from several threads on the same plan (each call on its own stream) -- with
  * one exception: a plan that works in K slices (sddmm_plan_info.k_slice < K,
  * i.e. K > 128) keeps the partial results between its slices in a buffer of
- * its own, so executes of such a plan must not overlap in time.
+ * its own, so executes of such a plan must not overlap in time -- unless they
+ * are made through sddmm_execute_ws, which takes that memory from the caller.
  */
 #ifndef SDDMM_H
 #define SDDMM_H
@@ -215,9 +216,12 @@ int sddmm_plan_create_device(int64_t n_rows, int64_t n_cols, int64_t nnz, const 
  *
  * tile_size_x is honoured by every LDS-tile launch (capped by what fits the
  * 160 KB LDS).  tile_size_y is the row-panel height of the PANEL kernel and of
- * an explicitly requested LDS_TILE plan; the plans AUTO/HYBRID build assign
- * whole column tiles to workgroups and ignore it (plan_info.tile_size_y reports
- * INT32_MAX there).                                                          */
+ * an explicitly requested LDS_TILE plan, and, in the plans AUTO/HYBRID build,
+ * the height of the row ranges a wide matrix is walked in (tile_runs = 2: the
+ * rows are cut into at least rows / tile_size_y ranges of equal nonzero count).
+ * Their other tile launches cut the rows into one block of equal nonzero count
+ * per die (or per workgroup share of a tile) whatever tile_size_y says.
+ * plan_info.tile_size_y reports the most rows any one block or range holds.   */
 typedef struct sddmm_plan_options {
     int32_t kernel;             /* SDDMM_KERNEL_*                                   [SDDMM_KERNEL]        */
     int32_t tile_size_x;        /* columns of S per LDS tile, 0 = choose            [SDDMM_TILE_X]        */
@@ -332,6 +336,26 @@ int sddmm_execute(const sddmm_plan *plan, const float *d_val, const float *d_W, 
 int sddmm_execute_epilogue(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
                            float *d_out, int32_t epilogue, void *stream);
 
+/* The same calls with the scratch memory brought by the caller.  A plan whose
+ * launches cover K in several slices keeps partial results between the slices, a
+ * launch with a matrix-core share packs its operands, and the softmax pass keeps
+ * per-chunk records: sddmm_execute, sddmm_execute_epilogue and
+ * sddmm_execute_softmax hold that memory in the plan (or, for the softmax
+ * records, in a per-device array of the library), so two of their calls on one
+ * plan must not overlap in time unless the plan needs none (one launch over all
+ * of K, no softmax).  sddmm_execute_ws takes it from d_workspace instead --
+ * device memory, 256-byte aligned, at least sddmm_plan_workspace_bytes(plan)
+ * long, which the call may overwrite entirely and needs only until its work on
+ * `stream` has finished -- and touches nothing of the plan: any number of calls
+ * on one plan, each with a workspace of its own, may run at the same time (other
+ * threads, other streams).  form = SDDMM_EPILOGUE_SCALE or _RESIDUAL, ored with
+ * SDDMM_FORM_SOFTMAX for the row softmax of the result.  No counterpart in the
+ * reference, whose sddmm_GPU allocates per call (sddmm.cu:38-73).              */
+#define SDDMM_FORM_SOFTMAX 0x100
+int sddmm_plan_workspace_bytes(const sddmm_plan *plan, int64_t *bytes);
+int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
+                     float *d_out, int32_t form, void *d_workspace, int64_t workspace_bytes, void *stream);
+
 /* The forms that surround an SDDMM where it is used as sparse attention or
  * in graph networks -- "SDDMM ... is a core of many machine learning
  * algorithms" (README.md:1); the reference itself stops at the sampled product.
@@ -386,7 +410,11 @@ int sddmm_gpu(const sddmm_plan *plan, const float *h_W, const float *h_H, float 
               float *kernel_ms);
 
 /* Plan-free SDDMM over a CSR pattern in device memory that allocates nothing:
- * no hipMalloc / hipFree and no allocating library routine on any call.  It has
+ * no hipMalloc / hipFree and no allocating library routine in the call.  The
+ * first call of a process on a device looks up the address of the library's
+ * fixed array and is the first launch of its kernels, which is when the runtime
+ * may load the code object and materialise that array: make one warm-up call per
+ * device outside any graph capture; after it, no call allocates.  It has
  * no counterpart in the reference (whose sddmm_GPU allocates and frees on every
  * call, sddmm.cu:38-73, 147-150); it is for callers that cannot allocate --
  * code under HIP graph capture, tight serving loops, harnesses that forbid

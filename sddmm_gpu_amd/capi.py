@@ -18,6 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libsddmm_hip.so")
 OK, ERR_ARG, ERR_IO, ERR_FORMAT, ERR_RANGE, ERR_UNSORTED, ERR_HIP, ERR_NOMEM = range(8)
 KERNEL_AUTO, KERNEL_ROW_GATHER, KERNEL_LDS_TILE, KERNEL_PANEL, KERNEL_HYBRID, KERNEL_DENSE_BLOCK = 0, 1, 2, 3, 4, 5
 EPILOGUE_SCALE, EPILOGUE_RESIDUAL = 0, 1
+FORM_SOFTMAX = 0x100
 
 
 class SddmmError(RuntimeError):
@@ -113,6 +114,8 @@ SIGNATURES = {
     "sddmm_execute": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sddmm_execute_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
     "sddmm_execute_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sddmm_plan_workspace_bytes": (c_int, [c_void_p, POINTER(c_int64)]),
+    "sddmm_execute_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
     "sddmm_row_softmax": (c_int, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sddmm_spmm_csr": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
@@ -337,6 +340,16 @@ class Plan:
     def execute_softmax(self, d_val, d_W, d_H, d_out, stream=0):
         check(lib().sddmm_execute_softmax(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out),
                                           c_void_p(stream or None)))
+
+    def workspace_bytes(self):
+        n = c_int64()
+        check(lib().sddmm_plan_workspace_bytes(self.h, byref(n)))
+        return n.value
+
+    def execute_ws(self, d_val, d_W, d_H, d_out, d_workspace, workspace_bytes, form=0, stream=0):
+        """sddmm_execute_ws: form = EPILOGUE_SCALE / EPILOGUE_RESIDUAL, ored with FORM_SOFTMAX."""
+        check(lib().sddmm_execute_ws(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out), c_int32(form),
+                                     c_void_p(d_workspace or None), c_int64(workspace_bytes), c_void_p(stream or None)))
 
     def execute_profiled(self, d_val, d_W, d_H, d_out, stream=0):
         n = c_int32()

@@ -26,10 +26,9 @@ static void usage()
             "  input          Matrix Market coordinate file (or a .bin written by --save-bin)\n"
             "  K              rank of W (rows x K) and H (cols x K)\n"
             "  tile_size_X    columns of S per LDS tile (0 = auto)\n"
-            "  tile_size_Y    row-panel height (0 = auto)\n"
-            "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
-            "                 (the default plan assigns whole column tiles to workgroups and ignores it;\n"
-            "                  it shapes --kernel panel and --kernel lds)\n"
+            "  tile_size_Y    row-panel height (0 = auto): rows per panel of --kernel panel and --kernel lds, rows per\n"
+            "                 row range where the default plan walks a wide matrix range by range; other default\n"
+            "                 plans cut the rows into one block per die, print that height and say so\n"
             "options:\n"
             "  --ref-order    positionals as the reference binary reads them: K tile_size_Y tile_size_X\n"
             "  --transpose    input is column-sorted: convert to the row-sorted transpose first\n"
@@ -173,6 +172,8 @@ int main(int argc, char **argv)
         CHECK(sddmm_plan_get_info(plan, &info));
         if (plan_loaded) fprintf(stderr, "sddmm: plan loaded from %s (%.1f ms)\n", plan_path(input).c_str(), info.plan_ms);
         printf("\nTilesize: X = %d, tilesize: Y = %d, TB: %d\n", info.tile_size_x, info.tile_size_y, info.block);
+        if (ty > 0 && (int64_t)info.tile_size_y > 2 * (int64_t)ty)
+            fprintf(stderr, "sddmm: tile_size_Y = %ld is not used by this plan (its row blocks hold up to %d rows)\n", ty, info.tile_size_y);
         std::vector<float> ms((size_t)runs);
         for (int r = 0; r < runs; ++r) CHECK(sddmm_gpu(plan, W.data(), H.data(), out.data(), &ms[r]));
         std::sort(ms.begin(), ms.end());

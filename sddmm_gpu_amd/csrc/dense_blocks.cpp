@@ -71,6 +71,9 @@ int find_dense_blocks(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t
     std::vector<BlockSel> selb((size_t)n_rb);
     std::vector<int32_t> keep(deg);
     const int nt = hw_threads();
+    // (every thread keeps two words per column: a wide matrix on a host with many threads would spend
+    // gigabytes here to learn that it has no dense core -- such a matrix goes without dense blocks)
+    if ((int64_t)n_cols * 8 * nt > ((int64_t)1 << 30)) return SDDMM_OK;
     std::vector<std::vector<int32_t>> cnt_t((size_t)nt), slot_t((size_t)nt);
     parallel_dynamic(n_rb, 1, [&](int64_t b, int64_t e, int t) {
         std::vector<int32_t> &cnt = cnt_t[(size_t)t], &slot = slot_t[(size_t)t];

@@ -7,6 +7,7 @@
 #include <unistd.h>
 #include "internal.hpp"
 #include "kernels.hpp"
+#include "build_id.h"
 
 using namespace sddmm;
 
@@ -57,6 +58,10 @@ struct Launch {
     int32_t fn_g = 0, fn_kpl = 0, fn_exact = 0, fn_gather = 0, fn_nwaves = 0;
     int32_t fn_nwm = 0;  // tile kernel: waves per workgroup that run the launch's matrix-core share (0: none)
     int32_t fused_slices = 0;  // sliced tile launch small enough that its K slices run inside one kernel launch
+    // Scratch memory of the launch (partial results between K slices; packed operands of the matrix-core share):
+    // sizes, and where each lies in a caller's workspace (sddmm_execute_ws); the plan's own copies are in ta
+    int64_t part_bytes = 0, hp_bytes = 0, wp_bytes = 0;
+    int64_t ws_part = 0, ws_hp = 0, ws_wp = 0;
 };
 
 struct sddmm_plan {
@@ -68,6 +73,7 @@ struct sddmm_plan {
     const int32_t *d_row_ptr = nullptr, *d_col = nullptr;
     float *d_val = nullptr;
     int32_t requested_kernel = 0;
+    int64_t ws_softmax = 0, ws_bytes = 0;  // workspace layout: the launches' scratch, then the softmax pass's records
     sddmm_plan_options options{};  // what the plan was built with, environment overrides applied
     ~sddmm_plan()
     {
@@ -602,7 +608,9 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
     // and each range is walked from top to bottom by a group of workgroups of one die that hold the
     // tiles the rows at the front touch.
     bool panel_local = false;
-    int pl_slots = 0;      // workgroups per row range
+    int pl_groups = 0;     // groups of workgroups per die
+    int pl_slots = 0;      // workgroups per group (a group works on one row range at a time)
+    int64_t block_rows_max = 0;  // most rows in one row block / row range of the 2-D assignment
     int64_t pl_sub = 0;    // batches per piece of an item
     // Short batches (see tile_variant_shorts): the last chunk of a (row, tile) run that holds at
     // most G/2 nonzeros is kept apart from the full chunks, and eight such chunks make a batch of
@@ -666,7 +674,13 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
             const int live = (int)((n_seg + (int64_t)rows.size() - 1) / (int64_t)rows.size());
             const int groups = live <= per_die ? per_die / live : 0;
             if (groups >= 1) {
-                const int want = 8 * groups;
+                // tile_size_y (rows per range) asks for more, lower ranges: the groups then take several
+                // ranges each, one after the other
+                int want = 8 * groups;
+                if (c.opt.tile_size_y > 0) {
+                    const int64_t ranges = ((int64_t)rows.size() + c.opt.tile_size_y - 1) / c.opt.tile_size_y;
+                    want = (int)std::min<int64_t>((int64_t)want * std::max<int64_t>(1, (ranges + want - 1) / want), 1 << 20);
+                }
                 make_cuts(want);
                 int64_t n_it = 0, n_ne = 0;
                 for (int32_t j = 0; j < T.n_tiles; ++j) {
@@ -682,6 +696,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                 if (live >= 2 && (c.opt.tile_runs == 2 || (double)n_seg > 1.5 * ((double)rows.size() + (double)(n_it - n_ne) * x))) {
                     shares = want;
                     panel_local = true;
+                    pl_groups = groups;
                     pl_slots = per_die / groups;
                     // (banded 2^20, K=512, ms per step by batches per wave and piece: 4 -> 4.37, 8 -> 4.25,
                     // 16 -> 4.24, 32 -> 4.27, 128 -> 4.44; whole tiles in runs of neighbours: 4.56)
@@ -691,6 +706,10 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                 }
             }
         }
+        if (grid2d)
+            for (int sh = 0; sh < shares; ++sh)
+                block_rows_max = std::max<int64_t>(block_rows_max, std::lower_bound(rows.begin(), rows.end(), cut[(size_t)sh + 1]) -
+                                                                   std::lower_bound(rows.begin(), rows.end(), cut[(size_t)sh]));
         auto seg_begin = [&](int32_t j, int64_t sg) { return (sg == T.active_ptr[j]) ? T.tile_ptr[j] : T.active_end[sg - 1]; };
         // Layout with short batches: an item (row block x tile) is a sequence of whole batches.  Its
         // runs are cut into chunks of G positions; a run's last chunk with at most G/2 nonzeros is a
@@ -901,14 +920,14 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                         items.push_back(item_of(sh, j));
                     }
             } else if (panel_local) {
-                // Range sh belongs to die sh % 8, group sh / 8.  Its items, in tile order, go to the
+                // Range sh belongs to die sh % 8, group (sh / 8) % pl_groups.  Its items, in tile order, go to the
                 // group's workgroup that is free first (time counted in stream positions).  The waves of
                 // a workgroup split an item into equal contiguous parts, so an item is handed over in
                 // pieces of pl_sub batches: the rows a workgroup touches at one time then lie close
                 // together.  Pieces of one tile follow each other on the same workgroup (staged once).
                 std::vector<std::vector<WorkItem>> seq((size_t)c.cus);
                 for (int sh = 0; sh < shares; ++sh) {
-                    const int die = sh % 8, base = (sh / 8) * pl_slots;
+                    const int die = sh % 8, base = ((sh / 8) % pl_groups) * pl_slots;
                     std::vector<int64_t> free_at((size_t)pl_slots, 0);
                     for (int32_t j : tiles_ne) {
                         const WorkItem it = item_of(sh, j);
@@ -1019,6 +1038,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
         c.P->owned.push_back({d_part, bytes, true});
         c.dev_bytes += (int64_t)bytes;
         a.part = d_part;
+        L.part_bytes = (int64_t)bytes;
         // A small launch costs about as much as its work: its K slices then run inside one kernel launch, every wave
         // over its own positions slice after slice (K=256, ms per step: bag-of-words 0.0328 -> 0.0309; recommender
         // shape at 1.1 M nonzeros 0.0381 -> 0.0345, at 5.3 M 0.1267 -> 0.1218).  Not for large streams, whose
@@ -1066,6 +1086,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
         c.P->owned.push_back({d_wp, wp_bytes, true});
         c.dev_bytes += (int64_t)(hp_bytes + wp_bytes);
         a.mf_hp = d_hp; a.mf_wp = d_wp; a.mf_rowinfo = d_ri; a.mf_rows = d_rows;
+        L.hp_bytes = (int64_t)hp_bytes; L.wp_bytes = (int64_t)wp_bytes;
         a.mf_groups = (int32_t)NG; a.mf_n_cb = (int32_t)n_cb;
         a.tile_bytes = (int32_t)((int64_t)x * ks * 4);
         L.fn_nwm = mf_nwm;
@@ -1090,7 +1111,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
     if (gather) L.grid = (int32_t)std::max<int64_t>(1, (np + 2047) / 2048);
     if (int rc = resolve_functions(L)) return rc;
     if (I) {
-        I->tile_size_x = x; I->tile_size_y = panel_rows; I->n_col_tiles = n_tiles_all;
+        I->tile_size_x = x; I->tile_size_y = grid2d ? (int32_t)std::min<int64_t>(block_rows_max, INT32_MAX) : panel_rows; I->n_col_tiles = n_tiles_all;
         I->n_row_panels = panel_local ? shares : n_panels; I->n_blocks = n_blocks; I->lanes_per_nnz = G; I->lds_bytes = L.lds;
         I->grid = L.grid; I->block = L.block; I->k_slice = ks;
     }
@@ -1249,6 +1270,21 @@ int add_panel(Ctx &c, const std::vector<int32_t> &rows, int ks, int32_t tile_x, 
     return SDDMM_OK;
 }
 
+// Lays the scratch memory of every launch, and the records of the softmax pass, out in one block a caller can
+// bring along (sddmm_execute_ws), each piece on a 256-byte boundary.
+void assign_workspace(sddmm_plan *P)
+{
+    int64_t at = 0;
+    auto take = [&](int64_t bytes) { const int64_t o = at; at += (bytes + 255) / 256 * 256; return o; };
+    for (Launch &L : P->launches) {
+        L.ws_part = take(L.part_bytes);
+        L.ws_hp = take(L.hp_bytes);
+        L.ws_wp = take(L.wp_bytes);
+    }
+    P->ws_softmax = take(row_softmax_workspace_bytes(P->info.nnz));
+    P->ws_bytes = at;
+}
+
 // Common plan builder from host CSR arrays.  d_*_borrowed != null: the device
 // already holds that array.
 int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_ptr_all, const int32_t *col_ind_all,
@@ -1284,7 +1320,9 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     int64_t nnz_part = nnz;
 
     hipDeviceProp_t prop;
-    HIP_TRY(hipGetDeviceProperties(&prop, 0));
+    int device = 0;
+    HIP_TRY(hipGetDevice(&device));
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
     Ctx c{P, n_rows, n_cols, nnz, row_ptr_all, col_ind_all, vals, K, prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256};
     c.opt = opt;
     P->options = opt;
@@ -1346,7 +1384,12 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
         (int64_t)n_rows * (K / 4) <= (int64_t)UINT32_MAX && (int64_t)n_cols * (K / 4) <= (int64_t)UINT32_MAX) {
         const double threshold = (double)(opt.dense_permille > 0 ? opt.dense_permille : 300) / 1000.0;
         const int64_t min_dense = opt.dense_min_nnz >= 0 ? opt.dense_min_nnz : std::max<int64_t>(nnz / 50, 1 << 20);
-        if (int rc = find_dense_blocks(n_rows, n_cols, nnz, row_ptr_all, col_ind_all, kDenseTile, threshold, min_dense, D)) return rc;
+        // (a host too short of memory for the search plans without dense blocks)
+        try {
+            if (int rc = find_dense_blocks(n_rows, n_cols, nnz, row_ptr_all, col_ind_all, kDenseTile, threshold, min_dense, D)) return rc;
+        } catch (const std::bad_alloc &) {
+            D = DenseBlocks{};
+        }
         if (D.n_dense > 0) {
             if (int rc = add_dense(c, D, vals)) return rc;
             row_ptr = D.rem_row_ptr.data(); col_ind = D.rem_col.data(); nnz_part = nnz - D.n_dense;
@@ -1475,6 +1518,7 @@ int make_plan(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *row_pt
     I.n_launches = 0;
     for (const Launch &L : P->launches) I.n_launches += (L.k_slice > 0 && L.k_slice < K && !L.fused_slices) ? K / L.k_slice : 1;
     I.device_bytes = c.dev_bytes;
+    assign_workspace(P);
     I.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     guard.p = nullptr;
     *out = P;
@@ -1593,8 +1637,9 @@ static int check_execute_args(const sddmm_plan *plan, const float *d_W, const fl
 }
 
 // Issues the kernels of one launch-list entry (one per K slice) on `stream`.
+// ws: the caller's workspace (null: the plan's own scratch memory)
 static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d_val, const float *d_W,
-                         const float *d_H, float *d_out, hipStream_t stream, int epilogue = SDDMM_EPILOGUE_SCALE)
+                         const float *d_H, float *d_out, hipStream_t stream, int epilogue = SDDMM_EPILOGUE_SCALE, char *ws = nullptr)
 {
     const int residual = epilogue == SDDMM_EPILOGUE_RESIDUAL;
     const sddmm_plan_info &I = plan->info;
@@ -1622,6 +1667,13 @@ static void issue_launch(const sddmm_plan *plan, const Launch &L, const float *d
         ta.sval = d_val ? nullptr : L.sval;
         ta.W = d_W; ta.H = d_H; ta.out = d_out;
         ta.nnz = (int32_t)I.nnz;
+        if (ws) {
+            if (ta.part) ta.part = reinterpret_cast<float *>(ws + L.ws_part);
+            if (ta.mf_groups > 0) {
+                ta.mf_hp = reinterpret_cast<const float4 *>(ws + L.ws_hp);
+                ta.mf_wp = reinterpret_cast<const float4 *>(ws + L.ws_wp);
+            }
+        }
         if (ta.mf_groups > 0) {  // the matrix-core share reads its operands from packed copies of H and of its W rows
             ta.k_off = 0;
             launch_mf_pack(ta, stream);
@@ -1679,7 +1731,37 @@ int sddmm_execute_softmax(const sddmm_plan *plan, const float *d_val, const floa
     if (int rc = sddmm_execute(plan, d_val, d_W, d_H, d_out, stream)) return rc;
     if (plan->info.nnz == 0) return SDDMM_OK;
     if (!plan->d_row_ptr) return fail(SDDMM_ERR_ARG, "sddmm_execute_softmax: the plan holds no row pointers");
-    return launch_row_softmax(plan->info.n_rows, plan->d_row_ptr, d_out, d_out, stream);
+    return launch_row_softmax(plan->info.n_rows, plan->d_row_ptr, d_out, d_out, stream, nullptr, 0);
+}
+
+int sddmm_plan_workspace_bytes(const sddmm_plan *plan, int64_t *bytes)
+{
+    if (!plan || !bytes) return fail(SDDMM_ERR_ARG, "sddmm_plan_workspace_bytes: NULL argument");
+    *bytes = plan->ws_bytes;
+    return SDDMM_OK;
+}
+
+int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H, float *d_out,
+                     int32_t form, void *d_workspace, int64_t workspace_bytes, void *stream)
+{
+    if (int rc = check_execute_args(plan, d_W, d_H, d_out, "sddmm_execute_ws")) return rc;
+    const int32_t epilogue = form & 0xff;
+    const bool softmax = (form & SDDMM_FORM_SOFTMAX) != 0;
+    if ((form & ~(0xff | SDDMM_FORM_SOFTMAX)) || (epilogue != SDDMM_EPILOGUE_SCALE && epilogue != SDDMM_EPILOGUE_RESIDUAL))
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_ws: unknown form %d", (int)form);
+    if (epilogue == SDDMM_EPILOGUE_RESIDUAL && !d_val && !plan->d_val && plan->info.nnz > 0)
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_ws: the residual val - dot needs values (d_val or plan-owned)");
+    if (plan->info.nnz == 0) return SDDMM_OK;
+    if (plan->ws_bytes > 0 && (!d_workspace || workspace_bytes < plan->ws_bytes))
+        return fail(SDDMM_ERR_ARG, "sddmm_execute_ws: the plan needs a workspace of %lld bytes (sddmm_plan_workspace_bytes)",
+                    (long long)plan->ws_bytes);
+    if ((uintptr_t)d_workspace & 255u) return fail(SDDMM_ERR_ARG, "sddmm_execute_ws: the workspace must be 256-byte aligned");
+    char *ws = static_cast<char *>(d_workspace);
+    for (const Launch &L : plan->launches) issue_launch(plan, L, d_val, d_W, d_H, d_out, (hipStream_t)stream, epilogue, ws);
+    HIP_TRY(hipGetLastError());
+    if (!softmax) return SDDMM_OK;
+    if (!plan->d_row_ptr) return fail(SDDMM_ERR_ARG, "sddmm_execute_ws: the plan holds no row pointers");
+    return launch_row_softmax(plan->info.n_rows, plan->d_row_ptr, d_out, d_out, stream, ws + plan->ws_softmax, plan->info.nnz);
 }
 
 int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
@@ -1720,10 +1802,45 @@ struct PlanFileHeader {
     uint64_t pattern_hash;
     uint64_t n_allocs, n_launches;
     uint64_t code_row_ptr, code_col, code_val;
-    char build[40];
+    char build[40];          // SDDMM_BUILD_ID of the library that wrote the file: a hash of its sources
+    uint64_t meta_checksum;  // over info, options, allocation sizes and launch table as they lie in the file
+    uint64_t data_checksum;  // over the arrays, in pieces of kPlanPiece bytes per allocation (see piece_hash)
 };
 constexpr char kPlanMagic[8] = {'S', 'D', 'D', 'M', 'M', 'P', 'L', 'N'};
-constexpr uint32_t kPlanVersion = 3;
+constexpr uint32_t kPlanVersion = 4;
+constexpr size_t kPlanPiece = (size_t)16 << 20;  // arrays are read, copied and check-summed in pieces of this size
+
+// Hash of one piece of an array: four interleaved multiply-add chains over its 8-byte words (so that a
+// thread runs at memory speed), folded with the piece's place in the file.  The file's checksum is the
+// wrapping sum of its pieces' hashes, whatever order they are read in.
+uint64_t piece_hash(const void *data, size_t n, uint64_t alloc, uint64_t piece)
+{
+    const unsigned char *b = (const unsigned char *)data;
+    uint64_t h[4] = {0x243f6a8885a308d3ull, 0x13198a2e03707344ull, 0xa4093822299f31d0ull, 0x082efa98ec4e6c89ull};
+    constexpr uint64_t kMul = 0x9e3779b97f4a7c15ull;
+    size_t i = 0;
+    for (; i + 32 <= n; i += 32) {
+        uint64_t w[4];
+        memcpy(w, b + i, 32);
+        for (int k = 0; k < 4; ++k) h[k] = (h[k] ^ w[k]) * kMul + (h[k] >> 29);
+    }
+    uint64_t tail[4] = {0, 0, 0, 0};
+    memcpy(tail, b + i, n - i);
+    for (int k = 0; k < 4; ++k) h[k] = (h[k] ^ tail[k]) * kMul + (h[k] >> 29);
+    uint64_t x = (uint64_t)n;
+    for (int k = 0; k < 4; ++k) x = mix64(x ^ h[k]);
+    return mix64(x ^ (alloc << 32) ^ piece);
+}
+
+// a launch descriptor read from a file must describe a launch this library could have planned
+bool launch_plausible(const Launch &L, int64_t nnz)
+{
+    const int64_t slack = 2 * nnz + (1 << 20);  // padded streams stay well below twice the nonzeros + per-item rounding
+    return L.fn_kind >= 1 && L.fn_kind <= 5 && L.grid > 0 && L.grid <= (1 << 24) && L.block >= 64 && L.block <= 1024 &&
+           L.block % 64 == 0 && L.lds >= 0 && L.lds <= kLdsMaxBytes && L.nnz >= 0 && L.nnz <= nnz && L.rows >= 0 &&
+           L.positions >= 0 && L.positions <= slack + 62 * nnz && L.k_slice >= 0 && L.fn_nwm >= 0 && L.fn_nwm <= 8 &&
+           L.ta.n_items >= 0 && L.ta.n_units >= 0 && L.ka.n_items >= 0 && L.ta.mf_groups >= 0 && L.ta.mf_n_cb >= 0;
+}
 constexpr uint64_t kScratchBit = 1ull << 63;
 constexpr uint64_t kBorrowedRowPtr = (1ull << 63) | 1, kBorrowedCol = (1ull << 63) | 2;
 
@@ -1793,8 +1910,9 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
         return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is not a plan file", path);
     h.build[sizeof h.build - 1] = 0;
     if (h.version != kPlanVersion || h.sizeof_launch != sizeof(Launch) || h.sizeof_info != sizeof(sddmm_plan_info) ||
-        h.sizeof_options != sizeof(sddmm_plan_options) || strncmp(h.build, sddmm_version(), sizeof h.build - 1) != 0)
-        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s was written by another build of the library (%s)", path, h.build);
+        h.sizeof_options != sizeof(sddmm_plan_options) || strncmp(h.build, SDDMM_BUILD_ID, sizeof h.build - 1) != 0)
+        return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s was written by another build of the library (%s, this one is %s)", path,
+                    h.build, SDDMM_BUILD_ID);
     if (h.n_rows != n_rows || h.n_cols != n_cols || h.nnz != nnz || h.K != K)
         return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s holds a plan for %lld x %lld, nnz %lld, K %d, not for %lld x %lld, nnz %lld, K %d",
                     path, (long long)h.n_rows, (long long)h.n_cols, (long long)h.nnz, h.K, (long long)n_rows, (long long)n_cols,
@@ -1819,17 +1937,26 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
     P->launches.resize((size_t)h.n_launches);
     if (h.n_launches && fread((void *)P->launches.data(), sizeof(Launch), P->launches.size(), f) != P->launches.size())
         return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is cut short", path);
+    {
+        uint64_t m = piece_hash(&P->info, sizeof P->info, 0, 0) + piece_hash(&P->options, sizeof P->options, 0, 1) +
+                     piece_hash(sizes.data(), sizes.size() * 8, 0, 2) +
+                     piece_hash((const void *)P->launches.data(), P->launches.size() * sizeof(Launch), 0, 3);
+        if (m != h.meta_checksum) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged (launch table checksum)", path);
+        for (const Launch &L : P->launches)
+            if (!launch_plausible(L, nnz)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged (launch descriptor)", path);
+    }
     // The arrays: pieces of 16 MiB are read (pread) by a few threads, each into its own pair of pinned
-    // staging buffers, and copied to the device on the thread's own stream as they arrive.
-    constexpr size_t kPiece = (size_t)16 << 20;
+    // staging buffers, check-summed there and copied to the device on the thread's own stream as they arrive.
+    constexpr size_t kPiece = kPlanPiece;
     const long data_at = ftell(f);
     if (data_at < 0) return fail(SDDMM_ERR_IO, "sddmm_plan_load: cannot seek in %s", path);
-    struct Piece { void *dst; uint64_t file_off; size_t n; };
+    struct Piece { void *dst; uint64_t file_off; size_t n; uint64_t alloc, piece; };
     std::vector<Piece> pieces;
     int64_t total = 0;
     {
-        uint64_t at = (uint64_t)data_at;
+        uint64_t at = (uint64_t)data_at, alloc = 0;
         for (uint64_t word : sizes) {
+            ++alloc;
             const bool scratch = (word & kScratchBit) != 0;
             const uint64_t bytes = word & ~kScratchBit;
             if (bytes == 0 || bytes > ((uint64_t)1 << 40)) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged", path);
@@ -1839,17 +1966,17 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
             total += (int64_t)bytes;
             if (scratch) continue;
             for (uint64_t off = 0; off < bytes; off += kPiece)
-                pieces.push_back({(char *)d + off, at + off, (size_t)std::min<uint64_t>(kPiece, bytes - off)});
+                pieces.push_back({(char *)d + off, at + off, (size_t)std::min<uint64_t>(kPiece, bytes - off), alloc, off / kPiece});
             at += bytes;
         }
     }
     const int n_readers = (int)std::max<size_t>(1, std::min<size_t>({(size_t)8, (size_t)hw_threads(), pieces.size()}));
     std::vector<int> reader_rc((size_t)n_readers, 0);  // 0 ok, 1 short read, 2 HIP error
+    std::vector<uint64_t> reader_sum((size_t)n_readers, 0);
     const int fd = fileno(f);
     {
         std::vector<std::thread> th;
-        for (int t = 0; t < n_readers; ++t)
-            th.emplace_back([&, t] {
+        auto reader = [&](int t) {
                 void *stage[2] = {nullptr, nullptr};
                 hipEvent_t done[2] = {nullptr, nullptr};
                 hipStream_t st = nullptr;
@@ -1867,6 +1994,7 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
                         got += (size_t)r;
                     }
                     if (got != pc.n) { reader_rc[(size_t)t] = 1; break; }
+                    reader_sum[(size_t)t] += piece_hash(stage[turn], pc.n, pc.alloc, pc.piece);
                     ok = hipMemcpyAsync(pc.dst, stage[turn], pc.n, hipMemcpyHostToDevice, st) == hipSuccess &&
                          hipEventRecord(done[turn], st) == hipSuccess;
                 }
@@ -1874,7 +2002,15 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
                 if (!ok && !reader_rc[(size_t)t]) reader_rc[(size_t)t] = 2;
                 for (int i = 0; i < 2; ++i) { if (stage[i]) (void)hipHostFree(stage[i]); if (done[i]) (void)hipEventDestroy(done[i]); }
                 if (st) (void)hipStreamDestroy(st);
-            });
+        };
+        // (a thread that cannot be started: its share is read by this one)
+        for (int t = 0; t < n_readers; ++t) {
+            try {
+                th.emplace_back(reader, t);
+            } catch (const std::system_error &) {
+                reader(t);
+            }
+        }
         for (auto &x : th) x.join();
     }
     for (int rc : reader_rc) {
@@ -1882,6 +2018,11 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
         if (rc == 2) return fail(SDDMM_ERR_HIP, "sddmm_plan_load: copying %s to the device failed", path);
     }
     HIP_TRY(hipDeviceSynchronize());
+    {
+        uint64_t sum = 0;
+        for (uint64_t x : reader_sum) sum += x;
+        if (sum != h.data_checksum) return fail(SDDMM_ERR_FORMAT, "sddmm_plan_load: %s is damaged (array checksum)", path);
+    }
     // pointers
     void *q = nullptr;
     std::vector<void *> fields;
@@ -1917,6 +2058,7 @@ int load_plan_file(const char *path, int64_t n_rows, int64_t n_cols, int64_t nnz
     P->requested_kernel = h.requested_kernel;
     P->pattern_hash = h.pattern_hash;
     P->info.device_bytes = total;
+    assign_workspace(P);
     P->info.plan_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     guard.p = nullptr;
     *out = P;
@@ -1937,7 +2079,7 @@ int sddmm_plan_save(const sddmm_plan *plan, const char *path)
         h.n_rows = plan->info.n_rows; h.n_cols = plan->info.n_cols; h.nnz = plan->info.nnz; h.K = plan->info.K;
         h.requested_kernel = plan->requested_kernel; h.pattern_hash = plan->pattern_hash;
         h.n_allocs = plan->owned.size(); h.n_launches = plan->launches.size();
-        strncpy(h.build, sddmm_version(), sizeof h.build - 1);
+        strncpy(h.build, SDDMM_BUILD_ID, sizeof h.build - 1);
         if (!encode_pointer(plan, plan->d_row_ptr, &h.code_row_ptr)) h.code_row_ptr = kBorrowedRowPtr;
         if (!encode_pointer(plan, plan->d_col, &h.code_col)) h.code_col = kBorrowedCol;
         if (!encode_pointer(plan, plan->d_val, &h.code_val)) return fail(SDDMM_ERR_ARG, "sddmm_plan_save: values outside the plan's memory");
@@ -1956,27 +2098,42 @@ int sddmm_plan_save(const sddmm_plan *plan, const char *path)
             for (auto &row : L.tfns) for (auto &fp : row) fp = nullptr;
         }
         HIP_TRY(hipDeviceSynchronize());  // a set_values still in flight has to land first
-        FILE *f = fopen(path, "wb");
-        if (!f) return fail(SDDMM_ERR_IO, "sddmm_plan_save: cannot create %s", path);
-        FileCloser fc{f};
-        bool ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(&plan->info, sizeof plan->info, 1, f) == 1 &&
-                  fwrite(&plan->options, sizeof plan->options, 1, f) == 1;
-        std::vector<uint64_t> sizes;  // (bit 63: scratch, no contents in the file)
-        for (const auto &o : plan->owned) sizes.push_back((uint64_t)o.bytes | (o.scratch ? kScratchBit : 0));
-        ok = ok && (sizes.empty() || fwrite(sizes.data(), 8, sizes.size(), f) == sizes.size());
-        ok = ok && (ls.empty() || fwrite((const void *)ls.data(), sizeof(Launch), ls.size(), f) == ls.size());
-        std::vector<char> buf;
-        for (const auto &o : plan->owned) {
-            if (o.scratch) continue;
-            constexpr size_t kPiece = (size_t)64 << 20;
-            for (size_t off = 0; ok && off < o.bytes; off += kPiece) {
-                const size_t n = std::min(kPiece, o.bytes - off);
-                buf.resize(n);
-                HIP_TRY(hipMemcpy(buf.data(), (const char *)o.p + off, n, hipMemcpyDeviceToHost));
-                ok = fwrite(buf.data(), 1, n, f) == n;
+        // written under a temporary name and renamed when complete: an interrupted save leaves no file under `path`
+        const std::string tmp = std::string(path) + ".tmp";
+        FILE *f = fopen(tmp.c_str(), "wb");
+        if (!f) return fail(SDDMM_ERR_IO, "sddmm_plan_save: cannot create %s", tmp.c_str());
+        struct Unlink { const std::string &p; bool armed = true; ~Unlink() { if (armed) (void)remove(p.c_str()); } } cleanup{tmp};
+        bool ok;
+        {
+            FileCloser fc{f};
+            std::vector<uint64_t> sizes;  // (bit 63: scratch, no contents in the file)
+            for (const auto &o : plan->owned) sizes.push_back((uint64_t)o.bytes | (o.scratch ? kScratchBit : 0));
+            h.meta_checksum = piece_hash(&plan->info, sizeof plan->info, 0, 0) + piece_hash(&plan->options, sizeof plan->options, 0, 1) +
+                              piece_hash(sizes.data(), sizes.size() * 8, 0, 2) +
+                              piece_hash((const void *)ls.data(), ls.size() * sizeof(Launch), 0, 3);
+            ok = fwrite(&h, sizeof h, 1, f) == 1 && fwrite(&plan->info, sizeof plan->info, 1, f) == 1 &&
+                 fwrite(&plan->options, sizeof plan->options, 1, f) == 1;
+            ok = ok && (sizes.empty() || fwrite(sizes.data(), 8, sizes.size(), f) == sizes.size());
+            ok = ok && (ls.empty() || fwrite((const void *)ls.data(), sizeof(Launch), ls.size(), f) == ls.size());
+            std::vector<char> buf;
+            uint64_t alloc = 0;
+            for (const auto &o : plan->owned) {
+                ++alloc;
+                if (o.scratch) continue;
+                for (size_t off = 0; ok && off < o.bytes; off += kPlanPiece) {
+                    const size_t n = std::min(kPlanPiece, o.bytes - off);
+                    buf.resize(n);
+                    HIP_TRY(hipMemcpy(buf.data(), (const char *)o.p + off, n, hipMemcpyDeviceToHost));
+                    h.data_checksum += piece_hash(buf.data(), n, alloc, off / kPlanPiece);
+                    ok = fwrite(buf.data(), 1, n, f) == n;
+                }
             }
+            // the header once more, now with the checksum of what followed it
+            ok = ok && fseek(f, 0, SEEK_SET) == 0 && fwrite(&h, sizeof h, 1, f) == 1 && fflush(f) == 0;
         }
-        if (!ok || fflush(f) != 0) return fail(SDDMM_ERR_IO, "sddmm_plan_save: write to %s failed", path);
+        if (!ok) return fail(SDDMM_ERR_IO, "sddmm_plan_save: write to %s failed", tmp.c_str());
+        if (rename(tmp.c_str(), path) != 0) return fail(SDDMM_ERR_IO, "sddmm_plan_save: cannot rename %s to %s", tmp.c_str(), path);
+        cleanup.armed = false;
     } catch (const std::exception &e) {
         return fail(SDDMM_ERR_NOMEM, "sddmm_plan_save: %s", e.what());
     }

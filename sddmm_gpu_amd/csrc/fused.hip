@@ -4,6 +4,7 @@
 // Both work on the sorted S directly (CSR pointers + one fp32 per nonzero), so they follow a
 // plan's sddmm_execute on the same stream without any re-ordering.
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include "internal.hpp"
 
 using namespace sddmm;
@@ -26,15 +27,17 @@ constexpr int kSmRowsMax = kSmChunk + 128;  // row pointers of a chunk kept in L
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
 
 // (m, sum) of the cut pieces: [2c] the row that began before chunk c, [2c + 1] the row that ends after
-// it.  8 + 4 MiB per device, held until the process ends; kernels name the arrays directly.  Softmax calls that
-// overlap in time on one device share it and must not (calls on one stream never do).
-static __device__ __align__(256) float2 g_softmax_rec[2 * kSmMaxChunks];
-static __device__ __align__(256) int2 g_softmax_rows[kSmMaxChunks];  // first and last row of each chunk
+// it; and the first and last row of each chunk.  The kernels take both arrays as arguments: a caller's
+// workspace (sddmm_execute_ws), or these file-scope arrays, 8 + 4 MiB per device, held until the process
+// ends -- softmax calls without a workspace that overlap in time on one device share them and must not
+// (calls on one stream never do).
+static __device__ __align__(256) float2 g_softmax_rec_store[2 * kSmMaxChunks];
+static __device__ __align__(256) int2 g_softmax_rows_store[kSmMaxChunks];  // first and last row of each chunk
 
 // First kernel: the first and the last row of every chunk, one thread per chunk (two binary searches of
 // row_ptr whose loads the other threads' searches hide).
 __global__ __launch_bounds__(256)
-void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows)
+void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int2 *__restrict__ g_softmax_rows)
 {
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
@@ -182,7 +185,8 @@ constexpr int kSmList16 = kSmChunk / (kSmByLane + 1) + 1, kSmList64 = kSmChunk /
               kSmListWg = kSmChunk / (kSmByWave + 1) + 1;
 
 __global__ __launch_bounds__(kSmBlock)
-void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out)
+void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                    float2 *g_softmax_rec, const int2 *__restrict__ g_softmax_rows)
 {
     __shared__ __align__(16) float buf[kSmChunk];
     __shared__ int32_t rows_lds[kSmRowsMax];
@@ -282,7 +286,7 @@ void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t
 
 // (m, sum) of row [rb, re) from the records of the chunks it spans: the last-slot record of its first
 // chunk, the first-slot records of the others; every wave of the workgroup computes the same pair.
-__device__ __forceinline__ float2 merged_record(int64_t rb, int64_t re)
+__device__ __forceinline__ float2 merged_record(const float2 *__restrict__ g_softmax_rec, int64_t rb, int64_t re)
 {
     const int lane = threadIdx.x & 63;
     const int64_t ca = rb / kSmChunk, cb = (re - 1) / kSmChunk;
@@ -318,7 +322,8 @@ __device__ __forceinline__ void scale_range(float *out, int64_t b, int64_t e, fl
 }
 
 __global__ __launch_bounds__(kSmBlock)
-void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, float *out)
+void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, float *out,
+                                    const float2 *__restrict__ g_softmax_rec, const int2 *__restrict__ g_softmax_rows)
 {
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
@@ -328,14 +333,14 @@ void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t
         const int64_t r0 = rr.x, r1 = rr.y;
         const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
         if (b0 < c0 || e0 > c1) {  // the chunk's first row is cut (it began before the chunk, or it fills it and goes on)
-            const float2 all = merged_record(b0, e0);
+            const float2 all = merged_record(g_softmax_rec, b0, e0);
             const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
             const float f = expf(mine.x - all.x) / all.y;
             const int64_t pb = max(b0, c0), pe = min(e0, c1);
             scale_range(out, pb, pe, f);
         }
         if (r1 != r0 && e1 > c1) {  // another row begins inside the chunk and ends after it
-            const float2 all = merged_record(b1, e1);
+            const float2 all = merged_record(g_softmax_rec, b1, e1);
             const float2 mine = g_softmax_rec[2 * c + 1];
             const float f = expf(mine.x - all.x) / all.y;
             scale_range(out, b1, c1, f);
@@ -466,14 +471,55 @@ int last_error(const char *who)
 
 namespace sddmm {
 
-int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream)
+// device addresses of the file-scope record arrays on the current device (looked up once per device)
+static int softmax_store(float2 **rec, int2 **rows)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static float2 *rec_of[kMaxDevices] = {};
+    static int2 *rows_of[kMaxDevices] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: no usable current device");
+    std::lock_guard<std::mutex> lock(mu);
+    if (!rec_of[dev]) {
+        void *a = nullptr, *b = nullptr;
+        if ((e = hipGetSymbolAddress(&a, HIP_SYMBOL(g_softmax_rec_store))) != hipSuccess ||
+            (e = hipGetSymbolAddress(&b, HIP_SYMBOL(g_softmax_rows_store))) != hipSuccess || !a || !b)
+            return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        rec_of[dev] = static_cast<float2 *>(a);
+        rows_of[dev] = static_cast<int2 *>(b);
+    }
+    *rec = rec_of[dev];
+    *rows = rows_of[dev];
+    return SDDMM_OK;
+}
+
+int64_t row_softmax_workspace_bytes(int64_t nnz)
+{
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    return ((n_chunks * 24 + 255) / 256) * 256;  // two float2 and one int2 per chunk
+}
+
+int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream, void *d_ws, int64_t nnz)
 {
     if (n_rows <= 0) return SDDMM_OK;
+    float2 *rec = nullptr;
+    int2 *rows = nullptr;
+    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] row pairs
+        const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+        rec = static_cast<float2 *>(d_ws);
+        rows = reinterpret_cast<int2 *>(rec + 2 * n_chunks);
+    } else if (int rc = softmax_store(&rec, &rows)) {
+        return rc;
+    }
     // (the entry count lives on the device: the grid is sized for the machine, the kernels stride over the chunks)
     const unsigned grid = 256 * 4;  // (33 KB of LDS per workgroup: four per compute unit)
-    hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows);
-    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out);
-    hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out);
+    hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+                       rec, (const int2 *)rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out,
+                       (const float2 *)rec, (const int2 *)rows);
     return last_error("sddmm_row_softmax");
 }
 
@@ -485,7 +531,7 @@ int sddmm_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x
 {
     if (n_rows < 0 || (n_rows > 0 && (!d_row_ptr || !d_x || !d_out))) return fail(SDDMM_ERR_ARG, "sddmm_row_softmax: bad arguments");
     if (n_rows >= INT32_MAX) return fail(SDDMM_ERR_RANGE, "sddmm_row_softmax: more than 2^31 - 2 rows");
-    return launch_row_softmax(n_rows, d_row_ptr, d_x, d_out, stream);
+    return launch_row_softmax(n_rows, d_row_ptr, d_x, d_out, stream, nullptr, 0);
 }
 
 int sddmm_spmm_csr(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr, const int32_t *d_col_ind,

@@ -47,8 +47,11 @@ void parallel_ranges(int64_t n, int64_t grain,
 // take in turn from a shared counter (for work of uneven cost per index).
 void parallel_dynamic(int64_t n, int64_t chunk, const std::function<void(int64_t, int64_t, int)> &f);
 
-// out[p] = softmax over the entries of p's row of x (out may be x), on `stream` (a hipStream_t)
-int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream);
+// out[p] = softmax over the entries of p's row of x (out may be x), on `stream` (a hipStream_t).  d_ws: device memory of
+// row_softmax_workspace_bytes(nnz) bytes for the pass's records, nnz the number of entries (d_row_ptr[n_rows]); null: the
+// library's own per-device arrays, which calls that overlap in time would share.
+int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream, void *d_ws, int64_t nnz);
+int64_t row_softmax_workspace_bytes(int64_t nnz);
 
 bool check_sorted(const sddmm_coo &S);
 // CSR row pointers of a sorted matrix (n_rows+1 entries).

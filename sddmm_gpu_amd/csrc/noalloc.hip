@@ -64,6 +64,7 @@ extern "C" int sddmm_csr_noalloc(int64_t n_rows, int64_t n_cols, int64_t nnz, co
                     (long long)nnz, (long long)kMaxNnz);
     if (n_rows >= INT32_MAX || n_cols >= INT32_MAX) return fail(SDDMM_ERR_RANGE, "sddmm_csr_noalloc: sizes beyond int32 offsets");
     if (nnz == 0) return SDDMM_OK;
+    if (n_rows == 0 || n_cols == 0) return fail(SDDMM_ERR_ARG, "sddmm_csr_noalloc: %lld nonzeros in an empty matrix", (long long)nnz);
     if (!d_row_ptr || !d_col_ind || !d_W || !d_H || !d_out) return fail(SDDMM_ERR_ARG, "sddmm_csr_noalloc: NULL device pointer");
     if ((((uintptr_t)d_W | (uintptr_t)d_H) & 15u) && K % 4 == 0)
         return fail(SDDMM_ERR_ARG, "sddmm_csr_noalloc: W and H must be 16-byte aligned");
@@ -77,6 +78,9 @@ extern "C" int sddmm_csr_noalloc(int64_t n_rows, int64_t n_cols, int64_t nnz, co
     hipStream_t s = (hipStream_t)stream;
     const int rows_grid = (int)std::min<int64_t>((n_rows + 255) / 256, 8192);
     hipLaunchKernelGGL(batch_rows_kernel, dim3(rows_grid), dim3(256), 0, s, d_row_ptr, (int32_t)n_rows, batch_row);
+    // (the second kernel reads what the first writes: it is not issued when the first could not be)
+    if (hipError_t e1 = hipGetLastError(); e1 != hipSuccess)
+        return fail(SDDMM_ERR_HIP, "sddmm_csr_noalloc: launch failed: %s", hipGetErrorString(e1));
 
     KArgs a{};
     a.col_ind = d_col_ind; a.val = d_val; a.W = d_W; a.H = d_H; a.out = d_out;

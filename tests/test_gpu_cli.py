@@ -89,3 +89,42 @@ def test_cli_column_sorted_input_and_errors(oracle, tmp_path):
     assert r.returncode != 0
     r = subprocess.run([CLI], capture_output=True, text=True, timeout=60)
     assert r.returncode == 2 and "usage" in r.stderr
+
+
+def test_cli_tile_size_y_shapes_the_row_ranges_of_a_wide_matrix(oracle, tmp_path):
+    """A banded matrix with more column tiles than workgroups is walked in row ranges; the
+    fourth positional sets their height, and the second output line prints the height in use."""
+    d = synth.make(5, 2.0 ** -3, K=128)
+    rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], rows, cols, vals)
+    mtx = tmp_path / "banded.bin"
+    S.write_bin(mtx)
+    K = 128
+    W = oracle.initial(d["n_rows"], K); H = oracle.initial(d["n_cols"], K)
+    cpu = oracle.sddmm_csr(d["row_ptr"].numpy(), cols, vals, W, H)
+    vec = tmp_path / "oracle.f32"
+    cpu.tofile(vec)
+    env = dict(os.environ, SDDMM_TILE_RUNS="2")
+    seen = {}
+    for ty in (0, 2048, 512):
+        r = subprocess.run([CLI, str(mtx), str(K), "0", str(ty), "--no-plan-file", "--check-against", str(vec)], capture_output=True,
+                           text=True, timeout=300, env=env)
+        assert r.returncode == 0, r.stderr + r.stdout
+        assert re.search(r"diff values in CPU and GPU: 0 ", r.stdout), r.stdout
+        m = re.search(r"Tilesize: X = (\d+), tilesize: Y = (\d+), TB: (\d+)", r.stdout)
+        assert m, r.stdout
+        seen[ty] = int(m.group(2))
+        if ty:
+            # (ranges hold equal shares of the nonzeros: the clipped rows at the matrix edges make the outer ones taller)
+            assert 0.9 * ty <= seen[ty] <= 1.7 * ty, (ty, seen)
+            assert "is not used by this plan" not in r.stderr
+    assert seen[0] > 2 * seen[2048] > 2 * seen[512], seen
+    # a plan that cuts the rows into one block per die says that it does not use the value
+    d3 = synth.make(3, 0.05, K=128)
+    S3 = capi.Coo.from_arrays(d3["n_rows"], d3["n_cols"], d3["row_ind"].numpy(), d3["col_ind"].numpy(), d3["val"].numpy())
+    p3 = tmp_path / "rec.bin"
+    S3.write_bin(p3)
+    r = subprocess.run([CLI, str(p3), "128", "0", "64", "--no-plan-file"], capture_output=True, text=True, timeout=300,
+                       env=dict(os.environ, SDDMM_SPLIT_MIN_NNZ="0", SDDMM_TILE_FEW_BLOCKS="0"))
+    assert r.returncode == 0, r.stderr + r.stdout
+    assert "tile_size_Y = 64 is not used by this plan" in r.stderr, r.stderr

@@ -55,7 +55,7 @@ def test_full_size(oracle, cfg, K):
     rep = parity_report(out[idx].cpu().numpy(), cpu, K, absp, f64=f64)
     record_parity(f"full size config {cfg} K={K} nnz={nnz} (sample of 400000)", rep)
     assert rep["violations"] == 0, rep
-    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"] + max(3, rep["cpu_vs_f64_strict"] // 4), rep
+    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"], rep
     del W, H
 
     # (1b) values kept by the plan in stream order: the same arithmetic, so the same bits

@@ -277,3 +277,62 @@ def test_concurrent_executes_on_one_plan_and_concurrent_plan_creation(oracle):
         p.execute(0, W.data_ptr(), H.data_ptr(), o.data_ptr())
         torch.cuda.synchronize()
         assert torch.equal(o, ref)
+
+
+@pytest.mark.parametrize("K,softmax", [(256, False), (128, True), (256, True)])
+def test_concurrent_executes_with_caller_workspaces(oracle, K, softmax):
+    """sddmm_execute_ws takes the scratch memory (partial results between K slices, softmax records) from
+    the caller: four threads run the same K-sliced plan at the same time, each with a workspace and a
+    stream of its own, and every output has the bits of a lone call."""
+    import threading
+    d = synth.make(3, 0.05, K=K, seed=23)
+    dev = torch.device(DEV)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    plan = S.plan(K, options=capi.PlanOptions.defaults(split_min_nnz=0, fuse_slices=0, ignore_env=1))
+    assert plan.info()["k_slice"] == 128
+    nbytes = plan.workspace_bytes()
+    assert nbytes > 0 and nbytes % 256 == 0
+    if K > 128:
+        assert nbytes >= 4 * plan.info()["padded_positions"]
+    W = d["W"].to(dev); H = d["H"].to(dev)
+    form = capi.FORM_SOFTMAX if softmax else 0
+    ref = torch.empty(d["nnz"], device=dev)
+    if softmax:
+        plan.execute_softmax(0, W.data_ptr(), H.data_ptr(), ref.data_ptr())
+    else:
+        plan.execute(0, W.data_ptr(), H.data_ptr(), ref.data_ptr())
+    torch.cuda.synchronize()
+    if not softmax:
+        check(d, ref.cpu().numpy(), oracle, K)
+    # too small a workspace, or none, is refused
+    with pytest.raises(capi.SddmmError) as e:
+        plan.execute_ws(0, W.data_ptr(), H.data_ptr(), ref.data_ptr(), 0, 0, form)
+    assert e.value.code == capi.ERR_ARG
+    n_threads, reps = 4, 6
+    outs = [torch.full((d["nnz"],), float("nan"), device=dev) for _ in range(n_threads)]
+    wss = [torch.full((nbytes // 4,), float("nan"), device=dev) for _ in range(n_threads)]
+    streams = [torch.cuda.Stream() for _ in range(n_threads)]
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(reps):
+                plan.execute_ws(0, W.data_ptr(), H.data_ptr(), outs[i].data_ptr(), wss[i].data_ptr(), nbytes, form, streams[i].cuda_stream)
+            streams[i].synchronize()
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    th = [threading.Thread(target=worker, args=(i,)) for i in range(n_threads)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not errors, errors
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o, ref)
+    # the residual epilogue through the same entry point
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute_ws(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), wss[0].data_ptr(), nbytes, capi.EPILOGUE_RESIDUAL)
+    torch.cuda.synchronize()
+    residual_ok(out.cpu().numpy(), d, oracle, K)

@@ -47,7 +47,7 @@ def check(d, out, oracle, K=None, label=None):
     rep = parity_report(out, cpu, K, absp, f64=f64)
     record_parity(label or f"{d.get('name', 'matrix')} {d['n_rows']}x{d['n_cols']} nnz={d['nnz']} K={K}", rep)
     assert rep["violations"] == 0, rep
-    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"] + max(3, rep["cpu_vs_f64_strict"] // 4), rep
+    assert rep["gpu_vs_f64_strict"] <= rep["cpu_vs_f64_strict"], rep
     # the GPU's tree-shaped sum must not be less accurate than the sequential CPU sum
     err_gpu = np.abs(out - f64).max(); err_cpu = np.abs(cpu - f64).max()
     assert err_gpu <= 2 * err_cpu + 1e-30, (err_gpu, err_cpu, rep)

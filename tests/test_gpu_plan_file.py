@@ -113,6 +113,36 @@ def test_mismatched_key_is_rejected(tmp_path):
         assert e.value.code == code
 
 
+def test_damaged_and_foreign_files_are_rejected(tmp_path):
+    """One flipped byte anywhere in the launch table or in the arrays, or the build id of another
+    library build, and the file is refused before anything is launched; nothing is left under the
+    plan's name by a save that could not finish."""
+    d = synth.make(3, 0.03, K=128)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    o = capi.PlanOptions.defaults(ignore_env=1, split_min_nnz=0)
+    path = tmp_path / "good.plan"
+    S.plan(128, options=o).save(path)
+    assert not os.path.exists(str(path) + ".tmp")
+    good = path.read_bytes()
+    assert S.load_plan(path, 128, options=o).info()["K"] == 128
+    n = len(good)
+    build_at = good.index(b"sddmm-")  # the build id inside the header
+    spots = {"launch table": 600, "arrays, early": n // 3, "arrays, late": n - 5, "checksum": build_at + 40 + 9,
+             "build id": build_at + 8}
+    for what, at in spots.items():
+        bad = bytearray(good)
+        bad[at] ^= 0x10
+        f = tmp_path / "bad.plan"
+        f.write_bytes(bytes(bad))
+        with pytest.raises(capi.SddmmError) as e:
+            S.load_plan(f, 128, options=o)
+        assert e.value.code == capi.ERR_FORMAT, what
+    # a save into a directory that does not exist fails cleanly
+    with pytest.raises(capi.SddmmError) as e:
+        S.plan(128, options=o).save(tmp_path / "no_such_dir" / "x.plan")
+    assert e.value.code == capi.ERR_IO
+
+
 def test_cli_saves_and_reloads_the_plan(oracle, tmp_path):
     d = synth.make(2, 0.5)
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())

@@ -1,6 +1,8 @@
 """sddmm_csr_noalloc (the entry point that allocates nothing) against the plan-based
 row-gather path it is a variant of: same kernel, so the outputs must agree bit for bit.
-Two calls in a row share the library's one device array, the second on a smaller input."""
+Two calls in a row share the library's one device array, the second on a smaller input.
+The allocation check looks at the steady state (the second call): the first call of a process
+on a device is where the runtime may load the code object and materialise the fixed array."""
 import gc
 
 import numpy as np
@@ -100,3 +102,7 @@ def test_rejects_sizes_beyond_the_fixed_array():
     with pytest.raises(capi.SddmmError) as e:
         capi.csr_noalloc(10, 10, (1 << 28) + 1, 8, 8, 0, 8, 16, 16, 16)
     assert e.value.code == capi.ERR_RANGE
+    # nonzeros in a matrix without rows: refused on the host, nothing is launched
+    with pytest.raises(capi.SddmmError) as e:
+        capi.csr_noalloc(0, 10, 5, 8, 8, 0, 8, 16, 16, 16)
+    assert e.value.code == capi.ERR_ARG
