@@ -327,6 +327,16 @@ def main():
         _, sp_ms, _ = time_steps(lambda st: capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp, ci, y.data_ptr(), K0,
                                                           d["H"].data_ptr(), Y.data_ptr(), st), n_steps, n_warm, torch, 30.0)
         plan.close()
+        # the same product on the plan's column tiles (spmm_stream = 1)
+        plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], d["row_ptr"].data_ptr(), d["col_ind"].data_ptr(), K0,
+                                         options=capi.PlanOptions.defaults(kernel=kernel, spmm_stream=1, **opt_fields))
+        sp_info = plan.info()
+        Y2 = torch.empty(d["n_rows"], K0, device=dev)
+        _, spp_ms, _ = time_steps(lambda st: plan.spmm(y.data_ptr(), d["H"].data_ptr(), Y2.data_ptr(), 0, 0, st), n_steps, n_warm, torch, 30.0)
+        torch.cuda.synchronize()
+        sp_diff = float((Y2 - Y).abs().max() / Y.abs().max().clamp_min(1e-30))
+        plan.close()
+        del Y2
         sm_bytes = 8.0 * d["nnz"] + 4.0 * (d["n_rows"] + 1)
         sp_bytes = 8.0 * d["nnz"] + 4.0 * (d["n_rows"] + 1) + 4.0 * K0 * (info["cols_touched"] + d["n_rows"])
         line["fused"] = {
@@ -335,6 +345,9 @@ def main():
             "sddmm_plus_softmax": {"ms": round(es_ms, 4)},
             "spmm_csr": {"ms": round(sp_ms, 4), "gflops": round(2.0 * d["nnz"] * K0 / (sp_ms * 1e6), 1), "alg_bytes": sp_bytes,
                          "alg_gbps": round(sp_bytes / (sp_ms * 1e6), 1), "hbm_frac": round(sp_bytes / (sp_ms * 1e6) / HBM_PEAK_GBPS, 4)},
+            "spmm_plan": {"ms": round(spp_ms, 4), "gflops": round(2.0 * d["nnz"] * K0 / (spp_ms * 1e6), 1), "runs": sp_info["spmm_runs"],
+                          "alg_gbps": round(sp_bytes / (spp_ms * 1e6), 1), "hbm_frac": round(sp_bytes / (spp_ms * 1e6) / HBM_PEAK_GBPS, 4),
+                          "max_diff_vs_csr_over_max": sp_diff, "plan_device_bytes": sp_info["device_bytes"]},
             "steps": n_steps}
         del x, y, Y
     if args.tile_sweep:

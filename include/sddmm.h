@@ -88,6 +88,7 @@ typedef struct sddmm_plan_info {
     int64_t dense_blocks; /* its 128 x 128 blocks */
     int64_t matrix_nnz;   /* nonzeros of the LDS_TILE launch computed by its matrix-core waves (counted in class_nnz[0]) */
     int64_t matrix_rows;  /* the rows they belong to */
+    int64_t spmm_runs;    /* (row, tile) runs of the product's tile stream, one partial row of Y each (0: not built) */
 } sddmm_plan_info;
 
 const char *sddmm_last_error(void);
@@ -255,6 +256,8 @@ typedef struct sddmm_plan_options {
     int32_t matrix_permille;    /* least fill of such a row, in 1/1000 of n_cols      [SDDMM_MATRIX_PERMILLE] */
     int32_t matrix_waves;       /* matrix-core waves per workgroup: 4 (next to 12
                                    vector waves) or 8 (next to 8)                     [SDDMM_MATRIX_WAVES]  */
+    int32_t spmm_stream;        /* 1: the plan also lays out its LDS_TILE launch for the product
+                                   Y = X H (sddmm_plan_spmm) on the same column tiles  [SDDMM_SPMM_STREAM]   */
     int32_t ignore_env;         /* 1: the environment is not consulted                                      */
     int64_t gather_slab_cols;   /* padded gather streams S in slabs of this many columns [SDDMM_GATHER_SLAB_COLS] */
     int64_t gather_panel_rows;  /* ... and, inside, in panels of this many listed rows   [SDDMM_GATHER_PANEL_ROWS] */
@@ -375,9 +378,22 @@ int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_
  * (d_Y: n_rows*K fp32, overwritten; rows without entries become 0), the product
  * that consumes the attention weights.  Rows that straddle the 256-entry chunks
  * the waves work in are completed with fp32 atomic adds, so their last bits can
- * differ from run to run.                                                    */
+ * differ from run to run.
+ *
+ * sddmm_plan_spmm: the same product behind the plan of its SDDMM.  A plan made
+ * with spmm_stream = 1 walks the rows of its LDS_TILE launch once more, as
+ * (row, tile) runs: a group of 8 lanes adds x[p] * (its slice of the H row, read
+ * from the column tile in LDS) over a run and writes one partial row; a second
+ * kernel adds the partial rows of every row; the plan's other rows gather their
+ * H rows as sddmm_spmm_csr does.  No atomics: the same bits on every call.  The
+ * partial rows (K floats per run; sddmm_plan_info.spmm_runs) live in the plan, or
+ * in d_workspace (NULL, or as for sddmm_execute_ws).  Other plans (and H or Y not
+ * 16-byte aligned) take the sddmm_spmm_csr path on the plan's pattern.  d_x: nnz
+ * fp32 in sorted order, e.g. the output of sddmm_execute_softmax.            */
 int sddmm_execute_softmax(const sddmm_plan *plan, const float *d_val, const float *d_W, const float *d_H,
                           float *d_out, void *stream);
+int sddmm_plan_spmm(const sddmm_plan *plan, const float *d_x, const float *d_H, float *d_Y, void *d_workspace,
+                    int64_t workspace_bytes, void *stream);
 int sddmm_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream);
 int sddmm_spmm_csr(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *d_row_ptr,
                    const int32_t *d_col_ind, const float *d_x, int32_t K, const float *d_H, float *d_Y,

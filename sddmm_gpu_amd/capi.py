@@ -35,7 +35,7 @@ class PlanInfo(C.Structure):
                 ("n_blocks", c_int64), ("device_bytes", c_int64), ("class_nnz", c_int64 * 3), ("class_rows", c_int64 * 3), ("padded_positions", c_int64),
                 ("short_batches", c_int64),
                 ("plan_ms", c_double), ("dense_nnz", c_int64), ("dense_blocks", c_int64), ("matrix_nnz", c_int64),
-                ("matrix_rows", c_int64)]
+                ("matrix_rows", c_int64), ("spmm_runs", c_int64)]
 
     def as_dict(self):
         return {f: (list(getattr(self, f)) if f.startswith("class_") else getattr(self, f)) for f, _ in self._fields_}
@@ -46,7 +46,7 @@ class PlanOptions(C.Structure):
     _fields_ = [(n, c_int32) for n in (
         "kernel", "tile_size_x", "tile_size_y", "k_slice", "tile_lanes", "tile_waves", "tile_assign", "tile_few_blocks",
         "tile_short_batches", "tile_deal", "tile_runs", "gather_lanes", "gather_padded", "gather_sink", "row_padded",
-        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "fuse_slices", "matrix_rows", "matrix_permille", "matrix_waves", "ignore_env")] + [(n, c_int64) for n in (
+        "unpadded_tile", "dense_blocks", "dense_permille", "dense_rb_group", "fuse_slices", "matrix_rows", "matrix_permille", "matrix_waves", "spmm_stream", "ignore_env")] + [(n, c_int64) for n in (
         "gather_slab_cols", "gather_panel_rows", "dense_min_nnz", "panel_bytes", "short_row_max", "stage_factor", "split_min_nnz")]
 
     @classmethod
@@ -116,6 +116,7 @@ SIGNATURES = {
     "sddmm_execute_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_workspace_bytes": (c_int, [c_void_p, POINTER(c_int64)]),
     "sddmm_execute_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
+    "sddmm_plan_spmm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "sddmm_row_softmax": (c_int, [c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sddmm_spmm_csr": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
     "sddmm_plan_launch_count": (c_int, [c_void_p, POINTER(c_int32)]),
@@ -350,6 +351,10 @@ class Plan:
         """sddmm_execute_ws: form = EPILOGUE_SCALE / EPILOGUE_RESIDUAL, ored with FORM_SOFTMAX."""
         check(lib().sddmm_execute_ws(self.h, c_void_p(d_val or None), c_void_p(d_W), c_void_p(d_H), c_void_p(d_out), c_int32(form),
                                      c_void_p(d_workspace or None), c_int64(workspace_bytes), c_void_p(stream or None)))
+
+    def spmm(self, d_x, d_H, d_Y, d_workspace=0, workspace_bytes=0, stream=0):
+        check(lib().sddmm_plan_spmm(self.h, c_void_p(d_x or None), c_void_p(d_H), c_void_p(d_Y), c_void_p(d_workspace or None),
+                                    c_int64(workspace_bytes), c_void_p(stream or None)))
 
     def execute_profiled(self, d_val, d_W, d_H, d_out, stream=0):
         n = c_int32()

@@ -62,6 +62,10 @@ struct Launch {
     // sizes, and where each lies in a caller's workspace (sddmm_execute_ws); the plan's own copies are in ta
     int64_t part_bytes = 0, hp_bytes = 0, wp_bytes = 0;
     int64_t ws_part = 0, ws_hp = 0, ws_wp = 0;
+    // the product Y = X H on this launch's tiles (spmm_stream = 1; sp_on == 0: not built)
+    SpmmArgs sa{};
+    int32_t sp_on = 0, sp_grid = 0, sp_nwaves = 16;  // (16 waves per workgroup: 1.54 against 1.59 ms with 12 on the recommender shape)
+    int64_t sp_part_bytes = 0, ws_sp_part = 0;
 };
 
 struct sddmm_plan {
@@ -205,7 +209,7 @@ void default_options(sddmm_plan_options &o)
     o.tile_short_batches = -1; o.tile_deal = -1; o.tile_runs = -1; o.fuse_slices = -1; o.gather_lanes = -1; o.gather_padded = -1;
     o.gather_sink = -1; o.row_padded = -1; o.unpadded_tile = -1; o.dense_blocks = -1; o.dense_permille = -1;
     o.dense_rb_group = -1; o.ignore_env = 0;
-    o.matrix_rows = -1; o.matrix_permille = -1; o.matrix_waves = -1;
+    o.matrix_rows = -1; o.matrix_permille = -1; o.matrix_waves = -1; o.spmm_stream = -1;
     o.gather_slab_cols = -1; o.gather_panel_rows = -1; o.dense_min_nnz = -1; o.panel_bytes = -1; o.short_row_max = -1; o.stage_factor = -1; o.split_min_nnz = -1;
 }
 
@@ -223,6 +227,7 @@ void apply_env_overrides(sddmm_plan_options &o)
     i32("SDDMM_ROW_PADDED", o.row_padded); i32("SDDMM_UNPADDED_TILE", o.unpadded_tile); i32("SDDMM_DENSE", o.dense_blocks);
     i32("SDDMM_DENSE_PERMILLE", o.dense_permille); i32("SDDMM_DENSE_RB_GROUP", o.dense_rb_group);
     i32("SDDMM_MATRIX_ROWS", o.matrix_rows); i32("SDDMM_MATRIX_PERMILLE", o.matrix_permille); i32("SDDMM_MATRIX_WAVES", o.matrix_waves);
+    i32("SDDMM_SPMM_STREAM", o.spmm_stream);
     i64("SDDMM_GATHER_SLAB_COLS", o.gather_slab_cols); i64("SDDMM_GATHER_PANEL_ROWS", o.gather_panel_rows); i64("SDDMM_DENSE_MIN_NNZ", o.dense_min_nnz); i64("SDDMM_PANEL_BYTES", o.panel_bytes);
     i64("SDDMM_SHORT_ROW_MAX", o.short_row_max); i64("SDDMM_STAGE_FACTOR", o.stage_factor);
     i64("SDDMM_SPLIT_MIN_NNZ", o.split_min_nnz);
@@ -244,6 +249,8 @@ int resolve_functions(Launch &L)
     }
     case 3: {
         const TileVariant tv{L.fn_g, L.fn_kpl};
+        if (L.sp_on && spmm_tile_set_lds(L.k_slice, L.sp_nwaves, L.k_slice * 4 * L.ta.tile_x) != 0)
+            return fail(SDDMM_ERR_HIP, "plan: cannot set up the tile kernel of the product Y = X H");
         if (L.fn_nwm > 0) {  // (a launch with a matrix-core share covers all of K: one form per value mode)
             for (int vm = 0; vm < 5; ++vm) {
                 L.tfns[vm][0] = tile_kernel_mf(vm, L.fn_nwaves, L.fn_nwm);
@@ -621,6 +628,15 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
     const bool deal_tiles = c.opt.tile_deal != 0;
     std::vector<uint32_t> btype;
     std::vector<WorkItem> items;
+    std::vector<std::pair<int, int32_t>> item_keys;  // (row block, tile) of each entry of items ((-1, -1): an empty turn)
+    // The product Y = X H on the same items (spmm_stream = 1; see SpmmArgs): built below, next to the items
+    const bool want_spmm = c.opt.spmm_stream > 0 && !gather && !c.orig && mf_nwm == 0 && spmm_tile_supported(ks);
+    struct SpmmHost {
+        std::vector<WorkItem> items;
+        std::vector<int32_t> b_off, b_p0, b_len, row_part_ptr, part_slot;
+        std::vector<uint16_t> cols;
+        bool built = false;
+    } sp;
     // Stream order: row panel by row panel (panel_rows consecutive rows of the list),
     // inside a panel column tile by column tile, inside a tile rows ascending.  A
     // (panel, tile) pair with nonzeros is a "unit"; workgroups that work on the units of
@@ -879,6 +895,84 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                 }
             });
         }
+        auto build_spmm = [&](const std::vector<std::pair<int, int32_t>> &keys) {
+            // Runs of every item, longest first, eight to a bundle.  A run's nonzeros are consecutive in the sorted
+            // S (one row, consecutive columns), so a group needs the position of the first only.
+            struct Run { int32_t p0, len, row, tile_base; };
+            const size_t ni = keys.size();
+            std::vector<std::vector<Run>> runs(ni);
+            std::vector<int64_t> n_bund(ni + 1, 0), n_blk(ni + 1, 0);
+            parallel_ranges((int64_t)ni, 1, [&](int64_t ib, int64_t ie, int) {
+                for (int64_t k = ib; k < ie; ++k) {
+                    const int sh = keys[(size_t)k].first;
+                    const int32_t j = keys[(size_t)k].second;
+                    if (sh < 0) continue;
+                    int64_t s0, s1;
+                    seg_range(sh, j, &s0, &s1);
+                    auto &rv = runs[(size_t)k];
+                    rv.reserve((size_t)(s1 - s0));
+                    for (int64_t sg = s0; sg < s1; ++sg) {
+                        const int64_t b = seg_begin(j, sg);
+                        rv.push_back({T.tiled_ind[(size_t)b], (int32_t)(T.active_end[(size_t)sg] - b), T.active_row[(size_t)sg],
+                                      (int32_t)((int64_t)j * x)});
+                    }
+                    std::stable_sort(rv.begin(), rv.end(), [](const Run &u, const Run &v) { return u.len > v.len; });
+                    const int64_t nb = ((int64_t)rv.size() + 7) / 8;
+                    int64_t blocks = 0;
+                    for (int64_t bb = 0; bb < nb; ++bb) blocks += (rv[(size_t)bb * 8].len + 7) / 8;  // rounds of 8 steps (the bundle's first run is its longest)
+                    n_bund[(size_t)k + 1] = nb;
+                    n_blk[(size_t)k + 1] = blocks;
+                }
+            });
+            for (size_t k = 0; k < ni; ++k) { n_bund[k + 1] += n_bund[k]; n_blk[k + 1] += n_blk[k]; }
+            const int64_t NB = n_bund[ni], NBLK = n_blk[ni];
+            if (NB * 8 < INT32_MAX && NBLK * 8 < INT32_MAX) {
+                sp.items.resize(ni);
+                sp.b_off.assign((size_t)NB + 1, 0);
+                sp.b_p0.assign((size_t)NB * 8, 0);
+                sp.b_len.assign((size_t)NB * 8, 0);
+                sp.cols.assign((size_t)NBLK * 64, 0);
+                sp.b_off[(size_t)NB] = (int32_t)NBLK;
+                // the rows' partial rows: counted per row, then listed
+                std::vector<int32_t> row_index((size_t)c.n_rows, -1);
+                for (size_t i = 0; i < rows.size(); ++i) row_index[(size_t)rows[i]] = (int32_t)i;
+                sp.row_part_ptr.assign(rows.size() + 1, 0);
+                for (size_t k = 0; k < ni; ++k)
+                    for (const Run &r : runs[k]) ++sp.row_part_ptr[(size_t)row_index[(size_t)r.row] + 1];
+                for (size_t i = 0; i < rows.size(); ++i) sp.row_part_ptr[i + 1] += sp.row_part_ptr[i];
+                sp.part_slot.assign((size_t)sp.row_part_ptr[rows.size()], 0);
+                std::vector<int32_t> fill_at(sp.row_part_ptr.begin(), sp.row_part_ptr.end() - 1);
+                for (size_t k = 0; k < ni; ++k) {  // (in item order: a row's partial rows are listed in the order they are written)
+                    const auto &rv = runs[k];
+                    for (size_t q = 0; q < rv.size(); ++q)
+                        sp.part_slot[(size_t)fill_at[(size_t)row_index[(size_t)rv[q].row]]++] = (int32_t)((n_bund[k] + (int64_t)q / 8) * 8 + (int64_t)q % 8);
+                }
+                parallel_ranges((int64_t)ni, 1, [&](int64_t ib, int64_t ie, int) {
+                    for (int64_t k = ib; k < ie; ++k) {
+                        const auto &rv = runs[(size_t)k];
+                        sp.items[(size_t)k] = {(int32_t)n_bund[(size_t)k], (int32_t)n_bund[(size_t)k + 1], 0,
+                                               keys[(size_t)k].second < 0 ? 0 : keys[(size_t)k].second};
+                        int64_t blk = n_blk[(size_t)k];
+                        for (int64_t bb = 0; bb * 8 < (int64_t)rv.size(); ++bb) {
+                            const int64_t B = n_bund[(size_t)k] + bb;
+                            const int n8 = (rv[(size_t)bb * 8].len + 7) / 8;
+                            sp.b_off[(size_t)B] = (int32_t)blk;
+                            for (int gq = 0; gq < 8 && bb * 8 + gq < (int64_t)rv.size(); ++gq) {
+                                const Run &r = rv[(size_t)(bb * 8 + gq)];
+                                sp.b_p0[(size_t)B * 8 + gq] = r.p0;
+                                sp.b_len[(size_t)B * 8 + gq] = r.len;
+                                for (int st = 0; st < n8 * 8; ++st) {  // (beyond the run: its last column again, with x = 0)
+                                    const int32_t p = r.p0 + std::min(st, r.len - 1);
+                                    sp.cols[((size_t)(blk + st / 8) * 8 + gq) * 8 + st % 8] = (uint16_t)(c.col_ind[p] - r.tile_base);
+                                }
+                            }
+                            blk += n8;
+                        }
+                    }
+                });
+                sp.built = true;
+            }
+        };
         if (grid2d) {
             std::vector<int32_t> tiles_ne;
             for (int32_t j = 0; j < T.n_tiles; ++j) if (T.active_ptr[j + 1] > T.active_ptr[j]) tiles_ne.push_back(j);
@@ -918,6 +1012,7 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                         const int sh = nt >= per_die ? die : die + 8 * (slot / nt);
                         const int32_t j = nt >= per_die ? deal[(size_t)die * nt + (size_t)step * per_die + slot] : slot % nt;
                         items.push_back(item_of(sh, j));
+                        item_keys.push_back({sh, j});
                     }
             } else if (panel_local) {
                 // Range sh belongs to die sh % 8, group (sh / 8) % pl_groups.  Its items, in tile order, go to the
@@ -964,11 +1059,20 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
                     for (int b = 0; b < c.cus; ++b) {
                         const int64_t idx = step * c.cus + (int64_t)(b % 8) * per_die + b / 8;
                         items.push_back(idx < n ? item_of(0, tiles_ne[(size_t)idx]) : WorkItem{0, 0, 0, 0});
+                        item_keys.push_back(idx < n ? std::pair<int, int32_t>{0, tiles_ne[(size_t)idx]} : std::pair<int, int32_t>{-1, -1});
                     }
             } else {
                 for (int sh = 0; sh < shares; ++sh)
-                    for (int32_t j : tiles_ne) items.push_back(item_of(sh, j));
+                    for (int32_t j : tiles_ne) { items.push_back(item_of(sh, j)); item_keys.push_back({sh, j}); }
             }
+            // the product walks the same (row block, tile) items on the same workgroups
+            if (want_spmm && !panel_local && item_keys.size() == items.size()) build_spmm(item_keys);
+        } else if (want_spmm && rb == 0 && rows.size() <= (size_t)panel_rows) {
+            // (equal position ranges for the SDDMM: the product takes one item per column tile)
+            std::vector<std::pair<int, int32_t>> keys;
+            for (int32_t j = 0; j < T.n_tiles; ++j)
+                if (T.active_ptr[j + 1] > T.active_ptr[j]) keys.push_back({0, j});
+            build_spmm(keys);
         }
     }
     unit_ptr.push_back((int32_t)np);
@@ -1092,6 +1196,45 @@ int add_tile(Ctx &c, const std::vector<int32_t> &rows_in, int32_t x, int32_t pan
         L.fn_nwm = mf_nwm;
         c.P->info.matrix_nnz += mf_nnz;
         c.P->info.matrix_rows += (int64_t)mf_rows.size();
+    }
+    if (sp.built) {
+        SpmmArgs &sa = L.sa;
+        WorkItem *d_it = nullptr;
+        int32_t *d_off = nullptr, *d_p0 = nullptr, *d_len = nullptr, *d_rpp = nullptr, *d_slot = nullptr, *d_sum = nullptr, *d_gat = nullptr;
+        uint16_t *d_cols = nullptr;
+        // the rows this launch does not hold (short ones, rows of other launches, rows without entries)
+        std::vector<int32_t> others;
+        {
+            size_t k = 0;
+            for (int64_t r = 0; r < c.n_rows; ++r) {
+                if (k < rows.size() && rows[k] == (int32_t)r) { ++k; continue; }
+                others.push_back((int32_t)r);
+            }
+            std::stable_sort(others.begin(), others.end(), [&](int32_t u, int32_t v) {
+                return c.row_ptr[u + 1] - c.row_ptr[u] > c.row_ptr[v + 1] - c.row_ptr[v];
+            });
+        }
+        if (int rc = c.up(&d_it, sp.items)) return rc;
+        if (int rc = c.up(&d_off, sp.b_off)) return rc;
+        if (int rc = c.up(&d_p0, sp.b_p0)) return rc;
+        if (int rc = c.up(&d_len, sp.b_len)) return rc;
+        if (int rc = c.up(&d_cols, sp.cols)) return rc;
+        if (int rc = c.up(&d_rpp, sp.row_part_ptr)) return rc;
+        if (int rc = c.up(&d_slot, sp.part_slot)) return rc;
+        if (int rc = c.up(&d_sum, rows)) return rc;
+        if (int rc = c.up(&d_gat, others)) return rc;
+        float *d_sp = nullptr;
+        const size_t bytes = sp.b_p0.size() * (size_t)ks * 4;
+        HIP_TRY(hipMalloc((void **)&d_sp, bytes));
+        c.P->owned.push_back({d_sp, bytes, true});
+        c.dev_bytes += (int64_t)bytes;
+        sa.items = d_it; sa.n_items = (int32_t)sp.items.size(); sa.b_off = d_off; sa.b_p0 = d_p0; sa.b_len = d_len; sa.cols = d_cols;
+        sa.part = d_sp; sa.row_part_ptr = d_rpp; sa.part_slot = d_slot; sa.sum_rows = d_sum; sa.n_sum_rows = (int64_t)rows.size();
+        sa.gather_rows = d_gat; sa.n_gather_rows = (int64_t)others.size();
+        sa.tile_x = x; sa.n_cols = (int32_t)c.n_cols; sa.K = c.K;
+        L.sp_on = 1; L.sp_part_bytes = (int64_t)bytes;
+        L.sp_grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (int64_t)sp.items.size()));
+        c.P->info.spmm_runs += (int64_t)sp.part_slot.size();
     }
     L.grid = (int32_t)std::max<int64_t>(1, std::min<int64_t>((int64_t)c.cus, (np + 4095) / 4096));
     if (grid2d) {
@@ -1280,6 +1423,7 @@ void assign_workspace(sddmm_plan *P)
         L.ws_part = take(L.part_bytes);
         L.ws_hp = take(L.hp_bytes);
         L.ws_wp = take(L.wp_bytes);
+        L.ws_sp_part = take(L.sp_part_bytes);
     }
     P->ws_softmax = take(row_softmax_workspace_bytes(P->info.nnz));
     P->ws_bytes = at;
@@ -1764,6 +1908,37 @@ int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_
     return launch_row_softmax(plan->info.n_rows, plan->d_row_ptr, d_out, d_out, stream, ws + plan->ws_softmax, plan->info.nnz);
 }
 
+int sddmm_plan_spmm(const sddmm_plan *plan, const float *d_x, const float *d_H, float *d_Y, void *d_workspace,
+                    int64_t workspace_bytes, void *stream)
+{
+    if (!plan) return fail(SDDMM_ERR_ARG, "sddmm_plan_spmm: plan is NULL");
+    const sddmm_plan_info &I = plan->info;
+    if (I.n_rows == 0) return SDDMM_OK;
+    if (!d_Y || (I.nnz > 0 && (!d_x || !d_H))) return fail(SDDMM_ERR_ARG, "sddmm_plan_spmm: NULL device pointer");
+    const Launch *Ls = nullptr;
+    for (const Launch &L : plan->launches)
+        if (L.sp_on) Ls = &L;
+    if (!Ls || ((((uintptr_t)d_H) | ((uintptr_t)d_Y)) & 15u)) {
+        // no tile stream for the product in this plan: the CSR form, gathering H rows
+        if (!plan->d_row_ptr || (I.nnz > 0 && !plan->d_col)) return fail(SDDMM_ERR_ARG, "sddmm_plan_spmm: the plan holds no pattern");
+        return sddmm_spmm_csr(I.n_rows, I.n_cols, I.nnz, plan->d_row_ptr, plan->d_col, d_x, I.K, d_H, d_Y, stream);
+    }
+    if (d_workspace) {
+        if (workspace_bytes < plan->ws_bytes) return fail(SDDMM_ERR_ARG, "sddmm_plan_spmm: the plan needs a workspace of %lld bytes", (long long)plan->ws_bytes);
+        if ((uintptr_t)d_workspace & 255u) return fail(SDDMM_ERR_ARG, "sddmm_plan_spmm: the workspace must be 256-byte aligned");
+    }
+    SpmmArgs sa = Ls->sa;
+    sa.x = d_x; sa.H = d_H; sa.Y = d_Y;
+    sa.row_ptr = plan->d_row_ptr; sa.col_ind = plan->d_col;
+    if (d_workspace) sa.part = reinterpret_cast<float *>(static_cast<char *>(d_workspace) + Ls->ws_sp_part);
+    for (int k_off = 0; k_off < I.K; k_off += Ls->k_slice) {
+        sa.k_off = k_off;
+        launch_spmm_slice(sa, Ls->k_slice, Ls->sp_nwaves, Ls->sp_grid, Ls->k_slice * 4 * Ls->ta.tile_x, stream);
+    }
+    HIP_TRY(hipGetLastError());
+    return SDDMM_OK;
+}
+
 int sddmm_plan_set_values(sddmm_plan *plan, const float *d_val, void *stream)
 {
     if (!plan) return fail(SDDMM_ERR_ARG, "sddmm_plan_set_values: plan is NULL");
@@ -1850,6 +2025,8 @@ void launch_pointer_fields(Launch &L, std::vector<void *> &fields)
     fields = {&L.ka.perm, &L.ka.scol, &L.ka.seg_row, &L.ka.batch_seg, &L.ka.batch_mask, &L.ka.items,
             &L.ta.perm, &L.ta.scol, &L.ta.grow, &L.ta.scol16, &L.ta.pbase, &L.ta.btype, &L.ta.part, &L.ta.sink, &L.ta.unit_ptr,
             &L.ta.unit_tile, &L.ta.items, &L.ta.mf_hp, &L.ta.mf_wp, &L.ta.mf_rowinfo, &L.ta.mf_rows,
+            &L.sa.items, &L.sa.b_off, &L.sa.b_p0, &L.sa.b_len, &L.sa.cols, &L.sa.part, &L.sa.row_part_ptr, &L.sa.part_slot,
+            &L.sa.sum_rows, &L.sa.gather_rows,
             &L.pa.slot_row, &L.pa.panel_tiles,
             &L.da.slot_rows, &L.da.slot_cols, &L.da.slot_range, &L.da.nz_p, &L.da.nz_rc,
             &L.sval, &L.perm};
@@ -1890,6 +2067,7 @@ bool same_options(const sddmm_plan_options &a, const sddmm_plan_options &b)
            a.row_padded == b.row_padded && a.unpadded_tile == b.unpadded_tile && a.dense_blocks == b.dense_blocks &&
            a.dense_permille == b.dense_permille && a.dense_rb_group == b.dense_rb_group &&
            a.matrix_rows == b.matrix_rows && a.matrix_permille == b.matrix_permille && a.matrix_waves == b.matrix_waves &&
+           a.spmm_stream == b.spmm_stream &&
            a.gather_slab_cols == b.gather_slab_cols && a.gather_panel_rows == b.gather_panel_rows &&
            a.dense_min_nnz == b.dense_min_nnz && a.panel_bytes == b.panel_bytes && a.short_row_max == b.short_row_max &&
            a.stage_factor == b.stage_factor && a.split_min_nnz == b.split_min_nnz;

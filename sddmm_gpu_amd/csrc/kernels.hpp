@@ -126,6 +126,31 @@ constexpr int kMfLdsPerWave = 512;     // ... and for each matrix-core wave's ro
 // packs the operands of the matrix-core share (a.mf_hp from a.H, a.mf_wp from a.W through a.mf_rows) on `stream`
 void launch_mf_pack(const TileArgs &a, void *stream);
 
+// Sparse-times-dense product Y = X H on a tile launch's column tiles (kernels_spmm.hip).  The rows of the
+// launch are walked as (row, tile) runs; eight runs of about equal length make a bundle, walked side by side
+// by the eight lane groups of a wave.
+struct SpmmArgs {
+    const WorkItem *items;     // per (row block, tile) item: [begin, end) = its bundles, tile = its column tile
+    int32_t n_items;
+    const int32_t *b_off;      // [n_bundles + 1] first round of each bundle (a round: 8 steps x 8 groups)
+    const int32_t *b_p0;       // [8 n_bundles] sorted position of each group's first nonzero (its run is consecutive there)
+    const int32_t *b_len;      // [8 n_bundles] nonzeros of each group's run (0: no run)
+    const uint16_t *cols;      // [rounds][8 groups][8 steps] column inside the tile (beyond the run: its last column again)
+    const float *x;            // [nnz] sorted order
+    const float *H;
+    float *part;               // [8 n_bundles][k slice] partial rows, one per run
+    float *Y;
+    const int32_t *row_part_ptr, *part_slot, *sum_rows;  // rows with runs: their partial rows (CSR-like) and their numbers
+    int64_t n_sum_rows;
+    const int32_t *gather_rows;  // the launch's other rows (gathered from global memory; rows without entries included)
+    int64_t n_gather_rows;
+    const int32_t *row_ptr, *col_ind;
+    int32_t tile_x, n_cols, K, k_off;
+};
+bool spmm_tile_supported(int k_slice);
+int spmm_tile_set_lds(int k_slice, int nwaves, int lds_bytes);  // 0 ok, 1 no such variant, 2 HIP error
+void launch_spmm_slice(const SpmmArgs &a, int k_slice, int nwaves, int grid, int lds_bytes, void *stream);
+
 // dst[i] = perm[i] >= 0 ? src[perm[i]] : 0 for i < n, on `stream` (a hipStream_t)
 void launch_gather_values(const int32_t *perm, const float *src, float *dst, int64_t n, void *stream);
 

@@ -160,3 +160,77 @@ def test_attention_chain_and_errors(oracle):
     with pytest.raises(capi.SddmmError) as e:
         capi.row_softmax(5, 0, att.data_ptr(), att.data_ptr())
     assert e.value.code == capi.ERR_ARG
+
+
+def spmm_ok(oracle, d, x, got, K):
+    want, absy = oracle.spmm_csr(d["row_ptr"].numpy(), d["col_ind"].numpy(), x.numpy(), d["H"].numpy(), with_abs=True)
+    assert np.all(np.isfinite(got))
+    deg = np.diff(d["row_ptr"].numpy()).astype(np.float64)
+    bound = 1e-5 * np.sqrt(np.maximum(deg, 1.0))[:, None] * absy + 1e-30
+    bad = np.abs(got.astype(np.float64) - want) > bound
+    assert not bad.any(), (int(bad.sum()), float(np.abs(got - want).max()))
+    assert np.all(got[deg == 0] == 0)
+
+
+@pytest.mark.parametrize("cfg,scale,K,opts", [
+    (3, 0.05, 128, {"split_min_nnz": 0}), (3, 0.05, 128, {"split_min_nnz": 0, "tile_few_blocks": 0}),
+    (3, 0.03, 256, {"split_min_nnz": 0}), (3, 0.03, 64, {"split_min_nnz": 0, "stage_factor": 0}), (3, 0.03, 32, {"split_min_nnz": 0, "stage_factor": 0}),
+    (2, 1.0, 256, {}), (2, 1.0, 128, {"tile_size_x": 192}), (5, 2.0 ** -6, 128, {}), (5, 2.0 ** -6, 512, {"tile_runs": 1}),
+    (1, 1.0, 32, {"kernel": capi.KERNEL_LDS_TILE})])
+def test_plan_spmm_on_the_tile_stream(oracle, cfg, scale, K, opts):
+    """Y = X H on the plan's column tiles (spmm_stream = 1): against the oracle, the same bits on
+    every call and with a caller's workspace, and the SDDMM of the same plan unchanged."""
+    d = synth.make(cfg, scale, K=K)
+    dev = torch.device(DEV)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    plan = S.plan(K, options=capi.PlanOptions.defaults(ignore_env=1, spmm_stream=1, **opts))
+    info = plan.info()
+    assert info["spmm_runs"] > 0, info
+    g = torch.Generator().manual_seed(K + cfg)
+    x = torch.randn(d["nnz"], generator=g)
+    xd = x.to(dev); H = d["H"].to(dev).contiguous(); W = d["W"].to(dev)
+    Y = torch.full((d["n_rows"], K), float("nan"), device=dev)
+    plan.spmm(xd.data_ptr(), H.data_ptr(), Y.data_ptr())
+    torch.cuda.synchronize()
+    spmm_ok(oracle, d, x, Y.cpu().numpy(), K)
+    Y2 = torch.full((d["n_rows"], K), float("nan"), device=dev)
+    plan.spmm(xd.data_ptr(), H.data_ptr(), Y2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Y2)
+    nbytes = plan.workspace_bytes()
+    assert nbytes >= 4 * K // max(1, K // info["k_slice"]) * info["spmm_runs"]
+    ws = torch.full((nbytes // 4,), float("nan"), device=dev)
+    Y3 = torch.full((d["n_rows"], K), float("nan"), device=dev)
+    plan.spmm(xd.data_ptr(), H.data_ptr(), Y3.data_ptr(), ws.data_ptr(), nbytes)
+    torch.cuda.synchronize()
+    assert torch.equal(Y, Y3)
+    # closed form: H of ones -> every output column is the row sum of x
+    ones = torch.ones_like(H)
+    plan.spmm(xd.data_ptr(), ones.data_ptr(), Y.data_ptr())
+    torch.cuda.synchronize()
+    deg = np.diff(d["row_ptr"].numpy()).astype(np.float64)
+    rs = np.bincount(d["row_ind"].numpy(), weights=x.numpy().astype(np.float64), minlength=d["n_rows"])
+    ab = np.bincount(d["row_ind"].numpy(), weights=np.abs(x.numpy()).astype(np.float64), minlength=d["n_rows"])
+    assert np.all(np.abs(Y.cpu().numpy()[:, K - 1] - rs) <= 1e-5 * np.sqrt(np.maximum(deg, 1.0)) * ab + 1e-30)
+    # the plan's SDDMM is what it was
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    from test_gpu_parity import check
+    check(d, out.cpu().numpy(), oracle, K)
+
+
+def test_plan_spmm_without_a_tile_stream_takes_the_csr_path(oracle):
+    K = 64
+    d = synth.make(3, 0.02, K=K)
+    dev = torch.device(DEV)
+    S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
+    x = torch.randn(d["nnz"], generator=torch.Generator().manual_seed(3))
+    xd = x.to(dev); H = d["H"].to(dev).contiguous()
+    for opts in ({}, {"kernel": capi.KERNEL_ROW_GATHER, "spmm_stream": 1}):
+        plan = S.plan(K, options=capi.PlanOptions.defaults(ignore_env=1, **opts))
+        assert plan.info()["spmm_runs"] == 0
+        Y = torch.full((d["n_rows"], K), float("nan"), device=dev)
+        plan.spmm(xd.data_ptr(), H.data_ptr(), Y.data_ptr())
+        torch.cuda.synchronize()
+        spmm_ok(oracle, d, x, Y.cpu().numpy(), K)
