@@ -94,19 +94,34 @@ void spmm_tile_kernel(const SpmmArgs a)
             for (int j = 0; j < KPL; ++j) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             for (int r = 0; r < n8; ++r) {
                 const Round q2 = fetch(h0, r + 2);
+                // the eight columns and values of the round, from the group's lanes; then the H pieces of step
+                // i + 1 are requested before the arithmetic of step i
+                int row_off[8];
+                float xs[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int src = (lane & ~7) + i;
-                    const int col = __shfl((int)q0.c, src);
-                    const float xs = __shfl(q0.x, src);
-                    const int row_off = col * (K4 * 16);
-                    const int addr_e = row_off + lane_e, addr_o = row_off + lane_o;
+                    row_off[i] = __shfl((int)q0.c, src) * (K4 * 16);
+                    xs[i] = __shfl(q0.x, src);
+                }
+                vec4f hb[2][KPL];
+                auto rd = [&](vec4f (&h)[KPL], int off) {
+                    const int addr_e = off + lane_e, addr_o = off + lane_o;
+#pragma unroll
+                    for (int j = 0; j < KPL; ++j) h[j] = *(lds_f4_ptr)(uintptr_t)(uint32_t)(((j & 1) ? addr_o : addr_e) + j * 128);
+                };
+                rd(hb[0], row_off[0]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (i + 1 < 8) rd(hb[(i + 1) & 1], row_off[i + 1]);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int j = 0; j < KPL; ++j) {
-                        const vec4f h = *(lds_f4_ptr)(uintptr_t)(uint32_t)(((j & 1) ? addr_o : addr_e) + j * 128);
-                        acc[j].x = fmaf(xs, h.x, acc[j].x); acc[j].y = fmaf(xs, h.y, acc[j].y);
-                        acc[j].z = fmaf(xs, h.z, acc[j].z); acc[j].w = fmaf(xs, h.w, acc[j].w);
+                        const vec4f h = hb[i & 1][j];
+                        acc[j].x = fmaf(xs[i], h.x, acc[j].x); acc[j].y = fmaf(xs[i], h.y, acc[j].y);
+                        acc[j].z = fmaf(xs[i], h.z, acc[j].z); acc[j].w = fmaf(xs[i], h.w, acc[j].w);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 q0 = q1; q1 = q2;
             }

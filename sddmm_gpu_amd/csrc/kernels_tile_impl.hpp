@@ -557,30 +557,49 @@ void sddmm_tile_kernel(const TileArgs a)
             float v = m.sv;
             if (SORTED_VAL) v = a.val[GATHER ? (m.p & 0x7fffffffu) : m.p];
             float acc[STEPS];
-            [&]<int... I>(std::integer_sequence<int, I...>) {
-                ((void)[&] {
-                    float s = 0.f;
-                    if constexpr (GATHER) {
+            if constexpr (!GATHER) {
+                // The H pieces of step I + 1 are requested before the arithmetic of step I, and the scheduler is kept
+                // from moving them back next to their use: an LDS read takes longer than the 16 multiply-adds of a
+                // step (same-box A/B, ms per step: recommender K = 128 0.835 -> 0.826, K = 256 1.702 -> 1.691,
+                // bag-of-words K = 256 0.0316 -> 0.0299; two steps ahead: no further gain).
+                vec4f hb[2][KPL];
+                auto rd = [&](vec4f (&h)[KPL], int cI) {
+                    int base[NB];  // cI is base 0 already
+                    base[0] = cI;
+#pragma unroll
+                    for (int t = 1; t < NB; ++t) base[t] = cI + base_step[t];
+#pragma unroll
+                    for (int j = 0; j < KPL; ++j) h[j] = *(lds_f4_ptr)(uintptr_t)(uint32_t)(base[j % NB] + j * G * 16);
+                };
+                rd(hb[0], c[0]);
+                [&]<int... I>(std::integer_sequence<int, I...>) {
+                    ((void)[&] {
+                        if constexpr (I + 1 < STEPS) rd(hb[(I + 1) & 1], c[I + 1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                        float s = 0.f;
+#pragma unroll
+                        for (int j = 0; j < KPL; ++j) {
+                            const vec4f h = hb[I & 1][j];
+                            s = dot4(w[j], make_float4(h.x, h.y, h.z, h.w), s);
+                        }
+                        acc[I] = s;
+                        __builtin_amdgcn_sched_barrier(0);
+                    }(), ...);
+                }(std::make_integer_sequence<int, STEPS>{});
+            } else {
+                [&]<int... I>(std::integer_sequence<int, I...>) {
+                    ((void)[&] {
                         const float4 *hr = H4 + (uint32_t)c[I];  // scol: float4 index of the H row
                         float4 h[KPL];
 #pragma unroll
                         for (int j = 0; j < KPL; ++j) h[j] = hr[slot[j]];
+                        float s = 0.f;
 #pragma unroll
                         for (int j = 0; j < KPL; ++j) s = dot4(w[j], h[j], s);
-                    } else {
-                        int base[NB];  // c[I] is base 0 already
-                        base[0] = c[I];
-#pragma unroll
-                        for (int t = 1; t < NB; ++t) base[t] = c[I] + base_step[t];
-#pragma unroll
-                        for (int j = 0; j < KPL; ++j) {
-                            const vec4f h = *(lds_f4_ptr)(uintptr_t)(uint32_t)(base[j % NB] + j * G * 16);
-                            s = dot4(w[j], make_float4(h.x, h.y, h.z, h.w), s);
-                        }
-                    }
-                    acc[I] = s;
-                }(), ...);
-            }(std::make_integer_sequence<int, STEPS>{});
+                        acc[I] = s;
+                    }(), ...);
+                }(std::make_integer_sequence<int, STEPS>{});
+            }
             columns_of_steps<G, XORDER>(next_col, lane_base0, cn);
             if constexpr (SHORT) {
                 transpose_reduce_step<G / 2, XORDER>(acc, l);  // inside each half group
