@@ -87,7 +87,7 @@ struct TileArgs {
     int32_t n_slices;    // the all-slices-in-one-launch form: K slices walked inside the launch, from k_off on
     // Matrix-core share of a launch (kernel variants with NWM > 0; mf_groups == 0: none).  The heaviest
     // rows, in groups of 32, are multiplied as whole 32 x 32 blocks against blocks of 32 consecutive
-    // columns by the last NWM waves of every workgroup, from operands packed by mf_pack_kernel:
+    // columns by the last NWM waves of every workgroup, from operands packed by sddmm_mf_pack_kernel:
     //   mf_hp[(cb * 32 + p) * 32 + j] = float4 p of the K slice of H row 32 cb + j (zero beyond n_cols)
     //   mf_wp[(g * 32 + p) * 32 + i]  = float4 p of the K slice of W row mf_rows[32 g + i]
     // (an MFMA operand load of one wave is then 1 KB of consecutive addresses).  Groups [die * G, (die + 1) * G),

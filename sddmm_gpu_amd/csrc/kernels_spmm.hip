@@ -23,7 +23,7 @@ typedef float vec4f __attribute__((ext_vector_type(4)));
 // KPL float4 per lane: a K slice of 32 * KPL elements on groups of 8 lanes
 template <int KPL, int NW>
 __global__ __launch_bounds__(NW * 64)
-void spmm_tile_kernel(const SpmmArgs a)
+void sddmm_spmm_tile_kernel(const SpmmArgs a)
 {
     extern __shared__ float4 lds_tile[];
     constexpr int G = 8, K4 = G * KPL;
@@ -140,7 +140,7 @@ void spmm_tile_kernel(const SpmmArgs a)
 // rows g, g + 8, ... and the groups' sums are added across the wave.
 template <int KPL>
 __global__ __launch_bounds__(256)
-void spmm_sum_kernel(const SpmmArgs a)
+void sddmm_spmm_sum_kernel(const SpmmArgs a)
 {
     constexpr int G = 8, K4 = G * KPL;
     const int lane = threadIdx.x & 63, l = lane & 7, g = lane >> 3;
@@ -179,7 +179,7 @@ void spmm_sum_kernel(const SpmmArgs a)
 // the rows longest first, so that the eight rows of a wave are about equally long.
 template <int KPL>
 __global__ __launch_bounds__(256)
-void spmm_rows_kernel(const SpmmArgs a)
+void sddmm_spmm_rows_kernel(const SpmmArgs a)
 {
     constexpr int G = 8;
     const int lane = threadIdx.x & 63, l = lane & 7;
@@ -236,7 +236,7 @@ bool spmm_tile_supported(int k_slice)
 int spmm_tile_set_lds(int k_slice, int nwaves, int lds_bytes)
 {
     const void *fn = nullptr;
-#define SDDMM_SPMM_FN(kpl) (nwaves == 12 ? (const void *)spmm_tile_kernel<kpl, 12> : (const void *)spmm_tile_kernel<kpl, 16>)
+#define SDDMM_SPMM_FN(kpl) (nwaves == 12 ? (const void *)sddmm_spmm_tile_kernel<kpl, 12> : (const void *)sddmm_spmm_tile_kernel<kpl, 16>)
     if (k_slice == 128) fn = SDDMM_SPMM_FN(4);
     else if (k_slice == 64) fn = SDDMM_SPMM_FN(2);
     else if (k_slice == 32) fn = SDDMM_SPMM_FN(1);
@@ -254,11 +254,11 @@ void launch_spmm_slice(const SpmmArgs &a, int k_slice, int nwaves, int grid, int
 #define SDDMM_SPMM_LAUNCH(kpl)                                                                                         \
     do {                                                                                                               \
         if (a.n_items > 0) {                                                                                           \
-            if (nwaves == 12) hipLaunchKernelGGL((spmm_tile_kernel<kpl, 12>), dim3((unsigned)grid), dim3(12 * 64), (size_t)lds_bytes, st, a); \
-            else hipLaunchKernelGGL((spmm_tile_kernel<kpl, 16>), dim3((unsigned)grid), dim3(16 * 64), (size_t)lds_bytes, st, a);              \
+            if (nwaves == 12) hipLaunchKernelGGL((sddmm_spmm_tile_kernel<kpl, 12>), dim3((unsigned)grid), dim3(12 * 64), (size_t)lds_bytes, st, a); \
+            else hipLaunchKernelGGL((sddmm_spmm_tile_kernel<kpl, 16>), dim3((unsigned)grid), dim3(16 * 64), (size_t)lds_bytes, st, a);              \
         }                                                                                                              \
-        if (a.n_sum_rows > 0) hipLaunchKernelGGL((spmm_sum_kernel<kpl>), dim3(sum_grid), dim3(256), 0, st, a);         \
-        if (a.n_gather_rows > 0) hipLaunchKernelGGL((spmm_rows_kernel<kpl>), dim3(rows_grid), dim3(256), 0, st, a);    \
+        if (a.n_sum_rows > 0) hipLaunchKernelGGL((sddmm_spmm_sum_kernel<kpl>), dim3(sum_grid), dim3(256), 0, st, a);         \
+        if (a.n_gather_rows > 0) hipLaunchKernelGGL((sddmm_spmm_rows_kernel<kpl>), dim3(rows_grid), dim3(256), 0, st, a);    \
     } while (0)
     if (k_slice == 128) SDDMM_SPMM_LAUNCH(4);
     else if (k_slice == 64) SDDMM_SPMM_LAUNCH(2);

@@ -9,7 +9,7 @@ namespace {
 // dst[(blk * 32 + p) * 32 + j] = float4 p of row j.  Reads are whole rows; the 16-byte writes of a
 // block fill its 16 KB.
 __global__ __launch_bounds__(256)
-void mf_pack_kernel(const float4 *__restrict__ src, const int32_t *__restrict__ rows, int32_t n_rows, int32_t row_k4,
+void sddmm_mf_pack_kernel(const float4 *__restrict__ src, const int32_t *__restrict__ rows, int32_t n_rows, int32_t row_k4,
                     int32_t k4_off, float4 *__restrict__ dst, int32_t n_blocks_first, const float4 *__restrict__ src2,
                     const int32_t *__restrict__ rows2, int32_t n_rows2, float4 *__restrict__ dst2)
 {
@@ -53,7 +53,7 @@ void launch_mf_pack(const TileArgs &a, void *stream)
 {
     const int row_k4 = a.K >> 2, k4_off = a.k_off >> 2;
     const int nb_h = a.mf_n_cb, nb_w = a.mf_groups;
-    hipLaunchKernelGGL(mf_pack_kernel, dim3((unsigned)(nb_h + nb_w)), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(sddmm_mf_pack_kernel, dim3((unsigned)(nb_h + nb_w)), dim3(256), 0, (hipStream_t)stream,
                        reinterpret_cast<const float4 *>(a.H), (const int32_t *)nullptr, a.n_cols, row_k4, k4_off,
                        const_cast<float4 *>(a.mf_hp), nb_h, reinterpret_cast<const float4 *>(a.W), a.mf_rows,
                        a.mf_groups * 32, const_cast<float4 *>(a.mf_wp));

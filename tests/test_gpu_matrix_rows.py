@@ -61,6 +61,14 @@ def test_matrix_rows_every_value_mode(oracle, waves, scale, permille):
     plan.execute(0, W.data_ptr(), H.data_ptr(), out3.data_ptr())
     torch.cuda.synchronize()
     assert torch.equal(out2, out3)
+    # the packed operands in a caller's workspace instead of the plan's
+    nbytes = plan.workspace_bytes()
+    assert nbytes >= 16384 * (info["matrix_rows"] // 32 + (d["n_cols"] + 31) // 32)
+    ws = torch.full((nbytes // 4,), float("nan"), device=dev)
+    out4 = torch.full((d["nnz"],), float("nan"), device=dev)
+    plan.execute_ws(0, W.data_ptr(), H.data_ptr(), out4.data_ptr(), ws.data_ptr(), nbytes)
+    torch.cuda.synchronize()
+    assert torch.equal(out4, out2)
     for src in (0, dv.data_ptr()):
         out.fill_(float("nan"))
         plan.execute_epilogue(src, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
