@@ -11,45 +11,73 @@ using namespace sddmm;
 
 namespace {
 
-// Row softmax in three kernels over equal chunks of the entries (not of the rows: a matrix may hold a few
-// rows of a million entries next to millions of rows of ten).  The first finds the rows at the ends of every chunk.  In the second a workgroup takes
-// kSmChunk consecutive entries into LDS and gives each of their rows to a lane, a group of lanes, a wave or
-// all its waves, by the row's length: maximum, sum of
-// exponentials, normalisation, all inside LDS; the chunk goes back to memory in one coalesced pass.  A row
-// that reaches beyond the chunk cannot be normalised yet: its piece is stored as exp(x - m) with the
-// piece's own maximum m, and (m, sum) goes into a record of the chunk.  The third kernel visits the chunks
-// again, merges the records of each cut row (at most two per chunk: the row that began before the chunk
-// and the row that ends after it) and scales the stored pieces.  Both kernels read the number of entries
+// Row softmax.  Every row is worked on whole wherever it fits on chip, so that an entry is read once
+// and written once, whatever the rows' lengths (a matrix may hold a few rows of a million entries next
+// to millions of rows of ten, so the work is cut by entries, not by rows):
+//   short rows (up to kSmChunk entries) are grouped into chunks of consecutive whole rows: chunk c
+//        starts with the row that holds entry c * kSmChunk and ends before the row that holds entry
+//        (c + 1) * kSmChunk, less than 2 * kSmChunk entries in all.  A workgroup takes a chunk into LDS
+//        and gives each row to a lane, a group of lanes, a wave or all its waves, by the row's length:
+//        maximum, sum of exponentials, normalisation, all inside LDS; the chunk goes back in one pass.
+//   long rows (up to kSmLongMax entries) belong to no chunk: one workgroup each holds the row in
+//        registers (the recommender shape keeps 56 % of its entries in rows of more than 4096).
+//   huge rows (beyond that) are cut at the multiples of kSmChunk: a piece is stored as exp(x - m) with the
+//        piece's own maximum m, (m, sum) goes into a record of the chunk, and a last kernel merges the
+//        records of each huge row and scales its pieces.
+// The first kernel lays the chunks out (one thread per chunk); all kernels read the number of entries
 // from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.
-constexpr int kSmChunk = 4096;  // (recommender / R-MAT, chunk + merge kernel in us: 2048 -> 367 + 196 / 767 + 357; 4096 -> 289 + 133 / 626 + 218; 8192 -> 371 + 124 / 889 + 171)
+constexpr int kSmChunk = 4096;
 constexpr int kSmBlock = 256;
-constexpr int kSmRowsMax = kSmChunk + 128;  // row pointers of a chunk kept in LDS at a time
+constexpr int kSmBuf = 2 * kSmChunk + 8;    // entries of a chunk in LDS: < 2 * kSmChunk, plus the float4 padding at both ends
+constexpr int kSmRowsMax = 1024 + 128;     // row pointers of a chunk kept in LDS at a time (with the buffers: 39 KB per workgroup)
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
+constexpr int kSmLongBlock = 256;                        // threads of a workgroup of the long-row kernel
+constexpr int kSmLongQ = 16;                             // float4 per thread
+constexpr int kSmLongMax = kSmLongQ * 4 * kSmLongBlock - 8;  // (less what a misaligned start costs)
 
-// (m, sum) of the cut pieces: [2c] the row that began before chunk c, [2c + 1] the row that ends after
-// it; and the first and last row of each chunk.  The kernels take both arrays as arguments: a caller's
-// workspace (sddmm_execute_ws), or these file-scope arrays, 8 + 4 MiB per device, held until the process
-// ends -- softmax calls without a workspace that overlap in time on one device share them and must not
-// (calls on one stream never do).
+__device__ __forceinline__ int softmax_row_class(int64_t len) { return len <= kSmChunk ? 0 : len <= kSmLongMax ? 1 : 2; }
+
+// (m, sum) of the pieces of huge rows: [2c] the row that began before chunk c, [2c + 1] the row that ends
+// after it; and the layout of each chunk: first entry, end, first row, last row.  The kernels take both
+// arrays as arguments: a caller's workspace (sddmm_execute_ws), or these file-scope arrays, 8 + 8 MiB per
+// device, held until the process ends -- softmax calls without a workspace that overlap in time on one
+// device share them and must not (calls on one stream never do).
 static __device__ __align__(256) float2 g_softmax_rec_store[2 * kSmMaxChunks];
-static __device__ __align__(256) int2 g_softmax_rows_store[kSmMaxChunks];  // first and last row of each chunk
+static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
 
-// First kernel: the first and the last row of every chunk, one thread per chunk (two binary searches of
-// row_ptr whose loads the other threads' searches hide).
+// First kernel: the layout, one thread per chunk (two binary searches of row_ptr whose loads the other
+// threads' searches hide).  With r the row that holds entry c * kSmChunk, chunk c begins at r's first
+// entry (r short), after r's last (r long: the long-row kernel owns it; the chunk may come out empty) or
+// at entry c * kSmChunk itself (r huge); it ends where chunk c + 1 would begin if that row were short
+// (so a long row that starts past the chunk's rows is left out) or at the multiple (huge).
 __global__ __launch_bounds__(256)
-void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int2 *__restrict__ g_softmax_rows)
+void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows)
 {
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t p0 = c * kSmChunk, p1 = min(nnz, p0 + kSmChunk) - 1;
+        const int64_t p0 = c * kSmChunk, p1 = min(nnz - 1, p0 + kSmChunk);  // (p1 = nnz - 1 in the last chunk: not used there)
         // first row whose end lies beyond p0 / p1
         int64_t lo0 = 0, hi0 = n_rows - 1, lo1 = 0, hi1 = n_rows - 1;
         while (lo0 < hi0 || lo1 < hi1) {
             if (lo0 < hi0) { const int64_t mid = (lo0 + hi0) >> 1; if (row_ptr[mid + 1] <= p0) lo0 = mid + 1; else hi0 = mid; }
             if (lo1 < hi1) { const int64_t mid = (lo1 + hi1) >> 1; if (row_ptr[mid + 1] <= p1) lo1 = mid + 1; else hi1 = mid; }
         }
-        g_softmax_rows[c] = make_int2((int)lo0, (int)lo1);
+        int4 lay;
+        const int64_t b0 = row_ptr[lo0], e0 = row_ptr[lo0 + 1];
+        const int k0 = softmax_row_class(e0 - b0);
+        lay.x = (int)(k0 == 0 ? b0 : k0 == 1 ? e0 : p0);
+        lay.z = (int)(k0 == 1 ? lo0 + 1 : lo0);
+        if (p0 + kSmChunk >= nnz) {
+            lay.y = (int)nnz;
+            lay.w = (int)(n_rows - 1);
+        } else {
+            const int64_t b1 = row_ptr[lo1], e1 = row_ptr[lo1 + 1];
+            const int k1 = softmax_row_class(e1 - b1);
+            lay.y = (int)(k1 == 2 ? p1 : b1);
+            lay.w = (int)(k1 == 2 ? lo1 : lo1 - 1);
+        }
+        g_softmax_rows[c] = lay;
     }
 }
 
@@ -80,89 +108,83 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
-// One row's piece buf[b, e) of a chunk: exp(x - max) in place and the sum; a whole row is normalised, a cut
-// row leaves (max, sum) in *rec.  Four forms, by how many lanes work on the row.
+// One row's piece buf[b, e) of a chunk: the lanes that work on it take it into registers (R entries
+// each, so that the LDS reads are all in flight together and the row is read and written once), maximum,
+// exp(x - max), sum; a whole row is normalised, a piece of a huge row is left as exp(x - max) with
+// (max, sum) in *rec.  Three forms, by how many lanes work on the row.
 
 // one lane (rows of a few entries: no lane exchanges at all)
 __device__ __forceinline__ void softmax_piece_by_lane(float *buf, int b, int e, bool whole, float2 *rec)
 {
-    float m = -INFINITY;
-    for (int i = b; i < e; ++i) m = fmaxf(m, buf[i]);
+    constexpr int R = 8;
+    float v[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) v[k] = b + k < e ? buf[b + k] : -INFINITY;
+    float m = v[0];
+#pragma unroll
+    for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
     float sum = 0.f;
-    for (int i = b; i < e; ++i) {
-        const float t = exp_nonpositive(buf[i] - m);
-        buf[i] = t;
-        sum += t;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        v[k] = b + k < e ? exp_nonpositive(v[k] - m) : 0.f;
+        sum += v[k];
     }
-    if (whole) {
-        const float inv = 1.0f / sum;
-        for (int i = b; i < e; ++i) buf[i] *= inv;
-    } else {
-        *rec = make_float2(m, sum);
-    }
+    const float f = whole ? 1.0f / sum : 1.0f;
+#pragma unroll
+    for (int k = 0; k < R; ++k) if (b + k < e) buf[b + k] = v[k] * f;
+    if (!whole) *rec = make_float2(m, sum);
 }
 
-// a group of GW lanes (all of them call this with the same row; the lane exchanges stay inside the group)
-template <int GW>
+// a group of GW lanes, up to GW * R entries (all lanes of the group call this with the same row; the lane
+// exchanges stay inside the group)
+template <int GW, int R>
 __device__ __forceinline__ void softmax_piece_by_group(float *buf, int b, int e, bool whole, float2 *rec)
 {
-    const int gl = threadIdx.x & (GW - 1);
-    // (four independent entries per round, so that the LDS reads of a long row overlap)
-    float m = -INFINITY;
-    int i = b + gl;
-    for (; i + 3 * GW < e; i += 4 * GW)
-        m = fmaxf(fmaxf(m, fmaxf(buf[i], buf[i + GW])), fmaxf(buf[i + 2 * GW], buf[i + 3 * GW]));
-    for (; i < e; i += GW) m = fmaxf(m, buf[i]);
+    const int i0 = b + (threadIdx.x & (GW - 1));
+    float v[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) v[k] = i0 + k * GW < e ? buf[i0 + k * GW] : -INFINITY;
+    float m = v[0];
+#pragma unroll
+    for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
     m = group_max<GW>(m);
     float sum = 0.f;
-    i = b + gl;
-    for (; i + 3 * GW < e; i += 4 * GW) {
-        const float t0 = exp_nonpositive(buf[i] - m), t1 = exp_nonpositive(buf[i + GW] - m),
-                    t2 = exp_nonpositive(buf[i + 2 * GW] - m), t3 = exp_nonpositive(buf[i + 3 * GW] - m);
-        buf[i] = t0; buf[i + GW] = t1; buf[i + 2 * GW] = t2; buf[i + 3 * GW] = t3;
-        sum += (t0 + t1) + (t2 + t3);
-    }
-    for (; i < e; i += GW) {
-        const float t = exp_nonpositive(buf[i] - m);
-        buf[i] = t;
-        sum += t;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        v[k] = i0 + k * GW < e ? exp_nonpositive(v[k] - m) : 0.f;
+        sum += v[k];
     }
     sum = group_sum<GW>(sum);
-    if (whole) {
-        const float inv = 1.0f / sum;
-        for (i = b + gl; i < e; i += GW) buf[i] *= inv;
-    } else if (gl == 0) {
-        *rec = make_float2(m, sum);
-    }
+    const float f = whole ? 1.0f / sum : 1.0f;
+#pragma unroll
+    for (int k = 0; k < R; ++k) if (i0 + k * GW < e) buf[i0 + k * GW] = v[k] * f;
+    if (!whole && i0 == b) *rec = make_float2(m, sum);
 }
 
-// the whole workgroup (every thread calls this with the same row).  red: 2 x (waves per workgroup) floats of LDS
+// the whole workgroup, up to kSmBlock * R entries (every thread calls this with the same row).
+// red: 2 x (waves per workgroup) floats of LDS
+template <int R>
 __device__ __forceinline__ void softmax_piece_by_workgroup(float *buf, float *red, int b, int e, bool whole, float2 *rec)
 {
     constexpr int NW = kSmBlock / 64;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float m = -INFINITY;
-    int i = b + threadIdx.x;
-    for (; i + 3 * kSmBlock < e; i += 4 * kSmBlock)
-        m = fmaxf(fmaxf(m, fmaxf(buf[i], buf[i + kSmBlock])), fmaxf(buf[i + 2 * kSmBlock], buf[i + 3 * kSmBlock]));
-    for (; i < e; i += kSmBlock) m = fmaxf(m, buf[i]);
+    const int i0 = b + threadIdx.x;
+    float v[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) v[k] = i0 + k * kSmBlock < e ? buf[i0 + k * kSmBlock] : -INFINITY;
+    float m = v[0];
+#pragma unroll
+    for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
     m = group_max<64>(m);
     if (lane == 0) red[wave] = m;
     __syncthreads();
 #pragma unroll
     for (int w = 0; w < NW; ++w) m = fmaxf(m, red[w]);
     float sum = 0.f;
-    i = b + threadIdx.x;
-    for (; i + 3 * kSmBlock < e; i += 4 * kSmBlock) {
-        const float t0 = exp_nonpositive(buf[i] - m), t1 = exp_nonpositive(buf[i + kSmBlock] - m),
-                    t2 = exp_nonpositive(buf[i + 2 * kSmBlock] - m), t3 = exp_nonpositive(buf[i + 3 * kSmBlock] - m);
-        buf[i] = t0; buf[i + kSmBlock] = t1; buf[i + 2 * kSmBlock] = t2; buf[i + 3 * kSmBlock] = t3;
-        sum += (t0 + t1) + (t2 + t3);
-    }
-    for (; i < e; i += kSmBlock) {
-        const float t = exp_nonpositive(buf[i] - m);
-        buf[i] = t;
-        sum += t;
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        v[k] = i0 + k * kSmBlock < e ? exp_nonpositive(v[k] - m) : 0.f;
+        sum += v[k];
     }
     sum = group_sum<64>(sum);
     if (lane == 0) red[NW + wave] = sum;
@@ -170,64 +192,90 @@ __device__ __forceinline__ void softmax_piece_by_workgroup(float *buf, float *re
     sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += red[NW + w];
-    if (whole) {
-        const float inv = 1.0f / sum;
-        for (i = b + threadIdx.x; i < e; i += kSmBlock) buf[i] *= inv;
-    } else if (threadIdx.x == 0) {
-        *rec = make_float2(m, sum);
-    }
+    const float f = whole ? 1.0f / sum : 1.0f;
+#pragma unroll
+    for (int k = 0; k < R; ++k) if (i0 + k * kSmBlock < e) buf[i0 + k * kSmBlock] = v[k] * f;
+    if (!whole && threadIdx.x == 0) *rec = make_float2(m, sum);
     // (the sums are read before the next row's second barrier, which comes after its first: no barrier needed here)
 }
 
 // piece lengths up to which a row is worked on by a lane / a group of 16 lanes / a wave; beyond: the workgroup
 constexpr int kSmByLane = 8, kSmBy16 = 192, kSmByWave = 1023;
-constexpr int kSmList16 = kSmChunk / (kSmByLane + 1) + 1, kSmList64 = kSmChunk / (kSmBy16 + 1) + 1,
-              kSmListWg = kSmChunk / (kSmByWave + 1) + 1;
+constexpr int kSmList16 = 2 * kSmChunk / (kSmByLane + 1) + 1, kSmList64 = 2 * kSmChunk / (kSmBy16 + 1) + 1,
+              kSmListWg = 2 * kSmChunk / (kSmByWave + 1) + 1;
 
-__global__ __launch_bounds__(kSmBlock)
+__global__ __launch_bounds__(kSmBlock, 3)  // (three waves per SIMD: 168 registers, a chunk ahead takes 36 of them)
 void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                    float2 *g_softmax_rec, const int2 *__restrict__ g_softmax_rows)
+                                    float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
 {
-    __shared__ __align__(16) float buf[kSmChunk];
+    __shared__ __align__(16) float buf[kSmBuf];
     __shared__ int32_t rows_lds[kSmRowsMax];
     __shared__ float red[2 * kSmBlock / 64];
     // rows of the chunk that take more than a lane, by class (index of the row inside the round's window)
     __shared__ uint16_t list16[kSmList16], list64[kSmList64], list_wg[kSmListWg];
     __shared__ int n_listed[3];
-    constexpr int kPer = kSmChunk / 4 / kSmBlock;  // float4 per thread and chunk
+    constexpr int kPer = (kSmBuf / 4 + kSmBlock - 1) / kSmBlock;  // float4 per thread and chunk, at most
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
-    // A whole chunk travels memory -> registers -> LDS; the registers are filled one chunk ahead, so the
-    // memory latency of chunk c + grid passes while chunk c is worked on.
-    float4 ahead[kPer];
-    int2 rows_ahead = make_int2(0, 0);
-    auto request = [&](int64_t c) {
-        if (c < n_chunks) rows_ahead = g_softmax_rows[c];
-        if (c < n_chunks && vec_in && (c + 1) * kSmChunk <= nnz) {
-            const float4 *src = reinterpret_cast<const float4 *>(x + c * kSmChunk);
+    // A chunk travels memory -> registers -> LDS as the float4 pieces from the aligned address below its
+    // first entry on; the registers are filled one chunk ahead, so the memory latency of chunk c + grid
+    // passes while chunk c is worked on.  The layout of a chunk says what to read, so the layouts are
+    // fetched two chunks ahead.
+    typedef float vec4 __attribute__((ext_vector_type(4)));  // (a plain vector: stays in registers through the conditional loads)
+    vec4 ahead[kPer];
+    auto layout_of = [&](int64_t c) { return c < n_chunks ? g_softmax_rows[c] : make_int4(0, 0, 0, 0); };
+    auto request = [&](int4 lay) __attribute__((always_inline)) {
+        if (vec_in && lay.x < lay.y) {
+            const int64_t a0 = lay.x & ~3;
+            const int nq = (int)((lay.y - a0 + 3) >> 2);
+            const vec4 *src = reinterpret_cast<const vec4 *>(x + a0);
 #pragma unroll
-            for (int u = 0; u < kPer; ++u) ahead[u] = src[threadIdx.x + u * kSmBlock];
+            for (int u = 0; u < kPer; ++u) {
+                const int q = threadIdx.x + u * kSmBlock;
+                // (the last float4 of the array may reach beyond its end: that one is read entry by entry below)
+                if (q < nq && a0 + 4 * (int64_t)q + 3 < nnz) ahead[u] = src[q];
+            }
         }
     };
-    request(blockIdx.x);
+    int4 lay_cur = layout_of(blockIdx.x), lay_nxt = layout_of((int64_t)blockIdx.x + gridDim.x);
+    request(lay_cur);
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int64_t c0 = c * kSmChunk, c1 = min(nnz, c0 + kSmChunk);
-        const int n = (int)(c1 - c0);
+        const int4 lay_after = layout_of(c + 2 * (int64_t)gridDim.x);
+        const int4 lay = lay_cur;
+        lay_cur = lay_nxt;
+        lay_nxt = lay_after;
+        if (lay.x >= lay.y) {  // no short or huge rows here
+            request(lay_cur);
+            continue;
+        }
+        const int64_t c0 = lay.x, c1 = lay.y;
+        const int64_t a0 = vec_in ? (c0 & ~(int64_t)3) : c0;  // buf[i] holds entry a0 + i
+        const int n = (int)(c1 - a0);
         __syncthreads();  // the chunk before has left the buffers
-        if (n == kSmChunk && vec_in) {
+        if (vec_in) {
+            const int nq = (n + 3) >> 2;
 #pragma unroll
-            for (int u = 0; u < kPer; ++u) reinterpret_cast<float4 *>(buf)[threadIdx.x + u * kSmBlock] = ahead[u];
+            for (int u = 0; u < kPer; ++u) {
+                const int q = threadIdx.x + u * kSmBlock;
+                if (q < nq) {
+                    if (a0 + 4 * (int64_t)q + 3 < nnz) {
+                        reinterpret_cast<vec4 *>(buf)[q] = ahead[u];
+                    } else {
+                        for (int j = 0; j < 4; ++j) buf[4 * q + j] = a0 + 4 * q + j < nnz ? x[a0 + 4 * q + j] : 0.f;
+                    }
+                }
+            }
         } else {
             for (int i0 = threadIdx.x; i0 < n; i0 += 8 * kSmBlock) {
                 float v[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = i0 + u * kSmBlock < n ? x[c0 + i0 + u * kSmBlock] : 0.f;
+                for (int u = 0; u < 8; ++u) v[u] = i0 + u * kSmBlock < n ? x[a0 + i0 + u * kSmBlock] : 0.f;
 #pragma unroll
                 for (int u = 0; u < 8; ++u) if (i0 + u * kSmBlock < n) buf[i0 + u * kSmBlock] = v[u];
             }
         }
-        const int64_t r0 = rows_ahead.x, r1 = rows_ahead.y;
+        const int64_t r0 = lay.z, r1 = lay.w;
         // The chunk's row pointers go into LDS, kSmRowsMax - 1 rows at a time (one round unless the chunk is
         // full of empty rows).  These loads are issued before the next chunk is requested, so that waiting
         // for them does not wait for it.
@@ -236,11 +284,13 @@ void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t
             if (w0 != r0) __syncthreads();  // the round before has left rows_lds and the lists
             for (int i = threadIdx.x; i <= n_w; i += kSmBlock) rows_lds[i] = row_ptr[w0 + i];
             if (threadIdx.x < 3) n_listed[threadIdx.x] = 0;
-            if (w0 == r0) request(c + gridDim.x);
+            if (w0 == r0) request(lay_cur);
             __syncthreads();
+            // (positions inside buf; only a huge row can reach beyond the chunk)
             auto piece = [&](int k, int *b, int *e, bool *whole, float2 **rec) {
                 const int64_t rb = rows_lds[k], re = rows_lds[k + 1];
-                *b = (int)(max(rb, c0) - c0); *e = (int)(min(re, c1) - c0);
+                *b = (int)(max(rb, c0) - a0); *e = (int)(min(re, c1) - a0);
+                if (softmax_row_class(re - rb) == 1) *e = *b;  // (no long row lies inside a chunk; should one, it is left alone)
                 *whole = rb >= c0 && re <= c1;
                 *rec = &g_softmax_rec[2 * c + (rb < c0 ? 0 : 1)];
             };
@@ -260,32 +310,169 @@ void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t
             for (int q = 0; q < n_wg; ++q) {
                 int b, e; bool whole; float2 *rec;
                 piece(list_wg[q], &b, &e, &whole, &rec);
-                softmax_piece_by_workgroup(buf, red, b, e, whole, rec);
+                if (e - b <= 8 * kSmBlock) softmax_piece_by_workgroup<8>(buf, red, b, e, whole, rec);
+                else softmax_piece_by_workgroup<kSmChunk / kSmBlock>(buf, red, b, e, whole, rec);
             }
             for (int q = threadIdx.x >> 6; q < n64; q += kSmBlock / 64) {
                 int b, e; bool whole; float2 *rec;
                 piece(list64[q], &b, &e, &whole, &rec);
-                softmax_piece_by_group<64>(buf, b, e, whole, rec);
+                if (e - b <= 6 * 64) softmax_piece_by_group<64, 6>(buf, b, e, whole, rec);
+                else softmax_piece_by_group<64, (kSmByWave + 63) / 64>(buf, b, e, whole, rec);
             }
             for (int q = threadIdx.x >> 4; q < n16; q += kSmBlock / 16) {
                 int b, e; bool whole; float2 *rec;
                 piece(list16[q], &b, &e, &whole, &rec);
-                softmax_piece_by_group<16>(buf, b, e, whole, rec);
+                if (e - b <= 4 * 16) softmax_piece_by_group<16, 4>(buf, b, e, whole, rec);
+                else softmax_piece_by_group<16, kSmBy16 / 16>(buf, b, e, whole, rec);
             }
         }
         __syncthreads();
-        if (n == kSmChunk && vec_out) {
-            float4 *dst = reinterpret_cast<float4 *>(out + c0);
+        const int lo = (int)(c0 - a0);  // 0 .. 3: the entries before belong to the chunk or the long row before
+        if (vec_in && vec_out) {
+            float4 *dst = reinterpret_cast<float4 *>(out + a0);
+            const int nq = (n + 3) >> 2;
 #pragma unroll
-            for (int u = 0; u < kPer; ++u) dst[threadIdx.x + u * kSmBlock] = reinterpret_cast<const float4 *>(buf)[threadIdx.x + u * kSmBlock];
+            for (int u = 0; u < kPer; ++u) {
+                const int q = threadIdx.x + u * kSmBlock, i = 4 * q;
+                if (q >= nq) continue;
+                if (i >= lo && i + 4 <= n) {
+                    dst[q] = reinterpret_cast<const float4 *>(buf)[q];
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) if (i + j >= lo && i + j < n) out[a0 + i + j] = buf[i + j];
+                }
+            }
         } else {
-            for (int i = threadIdx.x; i < n; i += kSmBlock) out[c0 + i] = buf[i];
+            for (int i = lo + threadIdx.x; i < n; i += kSmBlock) out[a0 + i] = buf[i];
         }
     }
 }
 
-// (m, sum) of row [rb, re) from the records of the chunks it spans: the last-slot record of its first
-// chunk, the first-slot records of the others; every wave of the workgroup computes the same pair.
+// One long row [rb, re) by a workgroup of kSmLongBlock threads, the row held in registers (4 * NQ floats
+// per thread): read once, written once.  x 16-byte aligned: float4 pieces counted from the aligned
+// address below the row's start (entries outside the row are masked); otherwise single entries, strided.
+template <int NQ>
+__device__ __forceinline__ void softmax_long_row(const float *x, float *out, int64_t rb, int64_t re, int64_t nnz, bool vec_in,
+                                                 bool vec_out, float *red)
+{
+    constexpr int NW = kSmLongBlock / 64;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    // (offsets relative to the aligned address below the row's start fit 32 bits)
+    const int64_t a0 = vec_in ? (rb & ~(int64_t)3) : rb;
+    const float *xr = x + a0;
+    float *outr = out + a0;
+    const int head = (int)(rb - a0), end = (int)(re - a0);
+    const int lim = (int)min(nnz - a0, (int64_t)INT32_MAX);  // entries of the array from a0 on
+    float f[4 * NQ];
+    if (vec_in) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k) {
+            const int p = 4 * (t + k * kSmLongBlock);
+            float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+            if (p < end) {
+                if (p + 3 < lim) {
+                    v = *reinterpret_cast<const float4 *>(xr + p);
+                } else {
+                    v.x = xr[p];
+                    if (p + 1 < lim) v.y = xr[p + 1];
+                    if (p + 2 < lim) v.z = xr[p + 2];
+                }
+            }
+            f[4 * k + 0] = (p + 0 >= head && p + 0 < end) ? v.x : -INFINITY;
+            f[4 * k + 1] = (p + 1 >= head && p + 1 < end) ? v.y : -INFINITY;
+            f[4 * k + 2] = (p + 2 >= head && p + 2 < end) ? v.z : -INFINITY;
+            f[4 * k + 3] = (p + 3 >= head && p + 3 < end) ? v.w : -INFINITY;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4 * NQ; ++k) {
+            const int p = t + k * kSmLongBlock;
+            f[k] = p < end ? xr[p] : -INFINITY;
+        }
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 4 * NQ; ++k) m = fmaxf(m, f[k]);
+    m = group_max<64>(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < NW; ++w) m = fmaxf(m, red[w]);
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4 * NQ; ++k) {
+        f[k] = f[k] == -INFINITY ? 0.f : exp_nonpositive(f[k] - m);
+        sum += f[k];
+    }
+    sum = group_sum<64>(sum);
+    if (lane == 0) red[NW + wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[NW + w];
+    const float inv = 1.0f / sum;
+    if (vec_in) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k) {
+            const int p = 4 * (t + k * kSmLongBlock);
+            if (p >= end) continue;
+            if (vec_out && p >= head && p + 4 <= end) {
+                *reinterpret_cast<float4 *>(outr + p) = make_float4(f[4 * k] * inv, f[4 * k + 1] * inv, f[4 * k + 2] * inv, f[4 * k + 3] * inv);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) if (p + j >= head && p + j < end) outr[p + j] = f[4 * k + j] * inv;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4 * NQ; ++k) {
+            const int p = t + k * kSmLongBlock;
+            if (p < end) outr[p] = f[k] * inv;
+        }
+    }
+    // (the next row writes its maxima after this row's second barrier and its sums after its own first: no barrier needed here)
+}
+
+// The long rows.  A long row holds the multiple of kSmChunk that follows its first entry, so it is the
+// row after the last row of the chunk whose window [c * kSmChunk, (c + 1) * kSmChunk) it starts in.
+// Workgroup b looks at the chunks b, b + grid, ...: first at many of them at once, a thread per chunk
+// (three dependent loads each, which a walk chunk by chunk would pay for one after the other), the long
+// rows that start in them collected in a list; then the list row by row.
+__global__ __launch_bounds__(kSmLongBlock, 4)  // (four waves per SIMD = 128 registers: four rows in flight per compute unit)
+void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                   const int4 *__restrict__ g_softmax_rows)
+{
+    __shared__ float red[2 * kSmLongBlock / 64];
+    __shared__ int2 todo[kSmLongBlock];
+    __shared__ int n_todo;
+    const int64_t nnz = row_ptr[n_rows];
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmLongBlock) {
+        __syncthreads();  // the list of the round before has been worked off
+        if (threadIdx.x == 0) n_todo = 0;
+        __syncthreads();
+        const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
+        if (c < n_chunks) {
+            const int64_t r = (int64_t)g_softmax_rows[c].w + 1;
+            if (r < n_rows) {
+                const int64_t rb = row_ptr[r], re = row_ptr[r + 1];
+                if (rb >= c * kSmChunk && rb < (c + 1) * kSmChunk && softmax_row_class(re - rb) == 1)
+                    todo[atomicAdd(&n_todo, 1)] = make_int2((int)rb, (int)re);
+            }
+        }
+        __syncthreads();
+        const int n = n_todo;
+        for (int q = 0; q < n; ++q) {
+            const int64_t rb = todo[q].x, re = todo[q].y;
+            if (re - rb <= 8 * 4 * kSmLongBlock - 8) softmax_long_row<8>(x, out, rb, re, nnz, vec_in, vec_out, red);
+            else softmax_long_row<kSmLongQ>(x, out, rb, re, nnz, vec_in, vec_out, red);
+        }
+    }
+}
+
+// (m, sum) of the huge row [rb, re) from the records of the chunks it spans: the last-slot record of its
+// first chunk, the first-slot records of the others; every wave of the workgroup computes the same pair.
 __device__ __forceinline__ float2 merged_record(const float2 *__restrict__ g_softmax_rec, int64_t rb, int64_t re)
 {
     const int lane = threadIdx.x & 63;
@@ -321,29 +508,54 @@ __device__ __forceinline__ void scale_range(float *out, int64_t b, int64_t e, fl
     }
 }
 
+// Last kernel: the pieces of huge rows are scaled to the whole row's maximum and sum.  A chunk holds at
+// most two of them: at its beginning (the row came from the chunk before, or fills this one and goes on)
+// and at its end.
 __global__ __launch_bounds__(kSmBlock)
 void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, float *out,
-                                    const float2 *__restrict__ g_softmax_rec, const int2 *__restrict__ g_softmax_rows)
+                                    const float2 *__restrict__ g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
 {
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int64_t c0 = c * kSmChunk, c1 = min(nnz, c0 + kSmChunk);
-        const int2 rr = g_softmax_rows[c];
-        const int64_t r0 = rr.x, r1 = rr.y;
-        const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
-        if (b0 < c0 || e0 > c1) {  // the chunk's first row is cut (it began before the chunk, or it fills it and goes on)
-            const float2 all = merged_record(g_softmax_rec, b0, e0);
-            const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
-            const float f = expf(mine.x - all.x) / all.y;
-            const int64_t pb = max(b0, c0), pe = min(e0, c1);
-            scale_range(out, pb, pe, f);
+    // (like the long-row kernel: the chunks are looked at many at a time, the few with work listed)
+    __shared__ int todo[kSmBlock];
+    __shared__ int n_todo;
+    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmBlock) {
+        __syncthreads();
+        if (threadIdx.x == 0) n_todo = 0;
+        __syncthreads();
+        {
+            const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
+            if (c < n_chunks) {
+                const int4 lay = g_softmax_rows[c];
+                if (lay.x < lay.y) {
+                    const int64_t r0 = lay.z, r1 = lay.w;
+                    if (softmax_row_class((int64_t)row_ptr[r0 + 1] - row_ptr[r0]) == 2 ||
+                        softmax_row_class((int64_t)row_ptr[r1 + 1] - row_ptr[r1]) == 2)
+                        todo[atomicAdd(&n_todo, 1)] = threadIdx.x;
+                }
+            }
         }
-        if (r1 != r0 && e1 > c1) {  // another row begins inside the chunk and ends after it
-            const float2 all = merged_record(g_softmax_rec, b1, e1);
-            const float2 mine = g_softmax_rec[2 * c + 1];
-            const float f = expf(mine.x - all.x) / all.y;
-            scale_range(out, b1, c1, f);
+        __syncthreads();
+        const int n = n_todo;
+        for (int q = 0; q < n; ++q) {
+            const int64_t c = base + (int64_t)todo[q] * gridDim.x;
+            const int4 lay = g_softmax_rows[c];
+            const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
+            const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
+            if (softmax_row_class(e0 - b0) == 2 && (b0 < c0 || e0 > c1)) {  // a huge row begins the chunk
+                const float2 all = merged_record(g_softmax_rec, b0, e0);
+                const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
+                const float f = expf(mine.x - all.x) / all.y;
+                const int64_t pb = max(b0, c0), pe = min(e0, c1);
+                scale_range(out, pb, pe, f);
+            }
+            if (r1 != r0 && softmax_row_class(e1 - b1) == 2 && e1 > c1) {  // another one begins inside the chunk and ends after it
+                const float2 all = merged_record(g_softmax_rec, b1, e1);
+                const float2 mine = g_softmax_rec[2 * c + 1];
+                const float f = expf(mine.x - all.x) / all.y;
+                scale_range(out, b1, c1, f);
+            }
         }
     }
 }
@@ -472,12 +684,12 @@ int last_error(const char *who)
 namespace sddmm {
 
 // device addresses of the file-scope record arrays on the current device (looked up once per device)
-static int softmax_store(float2 **rec, int2 **rows)
+static int softmax_store(float2 **rec, int4 **rows)
 {
     constexpr int kMaxDevices = 64;
     static std::mutex mu;
     static float2 *rec_of[kMaxDevices] = {};
-    static int2 *rows_of[kMaxDevices] = {};
+    static int4 *rows_of[kMaxDevices] = {};
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: no usable current device");
@@ -488,7 +700,7 @@ static int softmax_store(float2 **rec, int2 **rows)
             (e = hipGetSymbolAddress(&b, HIP_SYMBOL(g_softmax_rows_store))) != hipSuccess || !a || !b)
             return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
         rec_of[dev] = static_cast<float2 *>(a);
-        rows_of[dev] = static_cast<int2 *>(b);
+        rows_of[dev] = static_cast<int4 *>(b);
     }
     *rec = rec_of[dev];
     *rows = rows_of[dev];
@@ -498,28 +710,32 @@ static int softmax_store(float2 **rec, int2 **rows)
 int64_t row_softmax_workspace_bytes(int64_t nnz)
 {
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    return ((n_chunks * 24 + 255) / 256) * 256;  // two float2 and one int2 per chunk
+    return ((n_chunks * 32 + 255) / 256) * 256;  // two float2 and one int4 per chunk
 }
 
 int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream, void *d_ws, int64_t nnz)
 {
     if (n_rows <= 0) return SDDMM_OK;
     float2 *rec = nullptr;
-    int2 *rows = nullptr;
-    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] row pairs
+    int4 *rows = nullptr;
+    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] chunk layouts
         const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
         rec = static_cast<float2 *>(d_ws);
-        rows = reinterpret_cast<int2 *>(rec + 2 * n_chunks);
+        rows = reinterpret_cast<int4 *>(rec + 2 * n_chunks);
     } else if (int rc = softmax_store(&rec, &rows)) {
         return rc;
     }
     // (the entry count lives on the device: the grid is sized for the machine, the kernels stride over the chunks)
-    const unsigned grid = 256 * 4;  // (33 KB of LDS per workgroup: four per compute unit)
+    const unsigned grid = 256 * 4;
+    const unsigned grid_chunk = 256 * 3;  // (168 registers: three workgroups per compute unit)
     hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows);
-    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
-                       rec, (const int2 *)rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid_chunk), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+                       rec, (const int4 *)rows);
     hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out,
-                       (const float2 *)rec, (const int2 *)rows);
+                       (const float2 *)rec, (const int4 *)rows);
+    // (the long rows are touched by neither kernel above: this one could run anywhere after the first)
+    hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(2 * grid), dim3(kSmLongBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+                       (const int4 *)rows);
     return last_error("sddmm_row_softmax");
 }
 

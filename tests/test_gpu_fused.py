@@ -41,9 +41,9 @@ def test_row_softmax_matches_oracle(oracle, cfg, scale):
 
 @pytest.mark.parametrize("misalign", [0, 1])
 def test_row_softmax_edge_rows(oracle, misalign):
-    """Rows at the boundaries of the kernel's cases: entries are worked on in chunks of 4096; inside a chunk a row goes to
-    a lane (up to 8 entries), 16 lanes (up to 192), a wave (up to 1023) or the workgroup; a row cut by a chunk boundary is
-    finished by a second pass over the records of its pieces; a chunk's row pointers are staged 4223 rows at a time."""
+    """Rows at the boundaries of the kernel's cases: rows of up to 4096 entries are worked on in chunks of whole rows; inside
+    a chunk a row goes to a lane (up to 8 entries), 16 lanes (up to 192), a wave (up to 1023) or the workgroup; longer rows
+    have a kernel of their own (next test); a chunk's row pointers are staged 1151 rows at a time."""
     lens = ([0, 1, 0, 8, 9, 64, 65, 192, 193, 1023, 1024, 0, 2, 511]      # every class, whole rows
             + [4096 - sum([1, 8, 9, 64, 65, 192, 193, 1023, 1024, 2, 511])]  # ... up to the end of chunk 0 exactly
             + [4096]                                                        # a row that is exactly chunk 1
@@ -69,6 +69,46 @@ def test_row_softmax_edge_rows(oracle, misalign):
     capi.row_softmax(5, empty_rp.data_ptr(), xd.data_ptr(), out.data_ptr())
     torch.cuda.synchronize()
     assert bool(torch.isnan(obuf[:misalign]).all())  # (and nothing was written)
+
+
+@pytest.mark.parametrize("misalign", [0, 1, 2])
+def test_row_softmax_long_rows(oracle, misalign):
+    """Rows of more than a chunk (4096 entries) and up to 65,528 are held in registers by one workgroup each (up to
+    16,376 entries with 4 float4 per thread, beyond that with 16); longer ones go through the chunk records.  The cases:
+    the limits on both sides, a long row that starts exactly on a chunk boundary, long rows back to back, short rows
+    squeezed between them, a long row that ends the array (its last float4 is cut by the end of x)."""
+    lens = ([5, 4097, 3, 4096, 4098]                 # just over a chunk; a whole-chunk row is not long
+            + [4096 * 6 - (5 + 4097 + 3 + 4096 + 4098)]  # fill up to a chunk boundary ...
+            + [5000]                                 # ... so that this long row starts exactly on it
+            + [16376, 16377, 1, 0, 2]                # the two register classes
+            + [65528, 9000, 65529, 7]                # the longest long row, one after it, the shortest cut row
+            + [300] * 40 + [12345])                  # ordinary rows, and a long row at the end of the array
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    assert rp[-1] % 4 != 0  # (the array ends inside a float4)
+    rng = np.random.default_rng(2)
+    x = rng.normal(0, 6, rp[-1]).astype(np.float32)
+    x[rp[lens.index(65528)] + 60000] = 70.0; x[rp[lens.index(65529)] + 3] = 66.0; x[rp[-1] - 1] = 50.0
+    dev = torch.device(DEV)
+    xbuf = torch.zeros(len(x) + 8, device=dev); obuf = torch.full((len(x) + 8,), float("nan"), device=dev)
+    xd = xbuf[misalign:misalign + len(x)]; out = obuf[misalign:misalign + len(x)]
+    xd.copy_(torch.from_numpy(x))
+    rpd = torch.from_numpy(rp).to(dev)
+    capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    want = oracle.row_softmax(rp, x)
+    softmax_ok(out.cpu().numpy(), want)
+    assert bool(torch.isnan(obuf[:misalign]).all()) and bool(torch.isnan(obuf[misalign + len(x):]).all())  # nothing written outside
+    # in place; and input aligned with output not (and the other way round)
+    capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), xd.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(xd, out)
+    xd.copy_(torch.from_numpy(x))
+    other = torch.full((len(x) + 8,), float("nan"), device=dev)
+    o2 = other[3 - misalign:3 - misalign + len(x)]
+    capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), o2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(o2, out)
+    assert bool(torch.isnan(other[:3 - misalign]).all()) and bool(torch.isnan(other[3 - misalign + len(x):]).all())
 
 
 @pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])
