@@ -367,11 +367,14 @@ int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_
  * row-wise softmax of the results in place:
  *   out[p] = exp(s_p - m_r) / sum_{q in row r} exp(s_q - m_r),  s = val .* (W H^T) on S's pattern,
  * m_r the row's largest s.  One extra pass over out (the row totals must be known
- * before any entry can be normalised), made in equal chunks of entries whatever
- * the rows' lengths; a row cut by a chunk boundary is finished from per-chunk
- * (max, sum) records kept in a fixed device array of the library (12 MiB per
- * GPU), so softmax calls that overlap in time on one GPU (different streams or
- * threads) race; calls on one stream never do.
+ * before any entry can be normalised): every row of up to 16,376 entries is
+ * taken into registers whole -- by a lane, a group of lanes, a wave or a
+ * workgroup, by its length -- so it is read once and written once; a longer row
+ * is cut into pieces of 4096 entries whose (max, sum) records are merged by a
+ * last kernel.  The layout of the work and those records are kept in fixed
+ * device arrays of the library (16 MiB per GPU), so softmax calls that overlap
+ * in time on one GPU (different streams or threads) race unless they bring a
+ * workspace (sddmm_execute_ws); calls on one stream never do.
  * sddmm_row_softmax: the same pass on its own, over any CSR pattern in device
  * memory (d_out may be d_x; n_rows < 2^31 - 1, row_ptr[n_rows] entries).
  * sddmm_spmm_csr: Y[r, 0:K] = sum over row r's entries p of x[p] * H[col_p, 0:K]

@@ -11,29 +11,28 @@ using namespace sddmm;
 
 namespace {
 
-// Row softmax.  Every row is worked on whole wherever it fits on chip, so that an entry is read once
-// and written once, whatever the rows' lengths (a matrix may hold a few rows of a million entries next
-// to millions of rows of ten, so the work is cut by entries, not by rows):
+// Row softmax.  Every row is worked on whole, in registers, by as many lanes as its length asks for, so
+// that an entry is read once and written once whatever the rows' lengths (a matrix may hold a few rows of
+// a million entries next to millions of rows of ten, so the work is cut by entries, not by rows):
 //   short rows (up to kSmChunk entries) are grouped into chunks of consecutive whole rows: chunk c
 //        starts with the row that holds entry c * kSmChunk and ends before the row that holds entry
-//        (c + 1) * kSmChunk, less than 2 * kSmChunk entries in all.  A workgroup takes a chunk into LDS
-//        and gives each row to a lane, a group of lanes, a wave or all its waves, by the row's length:
-//        maximum, sum of exponentials, normalisation, all inside LDS; the chunk goes back in one pass.
-//   long rows (up to kSmLongMax entries) belong to no chunk: one workgroup each holds the row in
-//        registers (the recommender shape keeps 56 % of its entries in rows of more than 4096).
-//   huge rows (beyond that) are cut at the multiples of kSmChunk: a piece is stored as exp(x - m) with the
-//        piece's own maximum m, (m, sum) goes into a record of the chunk, and a last kernel merges the
-//        records of each huge row and scales its pieces.
+//        (c + 1) * kSmChunk.  A wave takes a chunk, 64 of its rows at a time: a lane per row of up to 8
+//        entries, then groups of 8 lanes (up to 96), of 32 lanes (up to 512), the whole wave (up to 1024
+//        in registers, beyond that in two walks over the row).
+//   long rows (up to kSmLongMax entries) belong to no chunk: a workgroup each (the recommender shape
+//        keeps 56 % of its entries in rows of more than 4096).
+//   huge rows (beyond that) are cut at the multiples of kSmChunk: a workgroup takes a piece, stores it
+//        as exp(x - m) with the piece's own maximum m and leaves (m, sum) in a record of the chunk; a last
+//        kernel merges the records of each huge row and scales its pieces.
 // The first kernel lays the chunks out (one thread per chunk); all kernels read the number of entries
-// from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.
+// from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.  No LDS staging: a
+// row's loads are all in flight together, and 16 waves per compute unit hide their latency.
 constexpr int kSmChunk = 4096;
 constexpr int kSmBlock = 256;
-constexpr int kSmBuf = 2 * kSmChunk + 8;    // entries of a chunk in LDS: < 2 * kSmChunk, plus the float4 padding at both ends
-constexpr int kSmRowsMax = 1024 + 128;     // row pointers of a chunk kept in LDS at a time (with the buffers: 39 KB per workgroup)
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
-constexpr int kSmLongBlock = 256;                        // threads of a workgroup of the long-row kernel
-constexpr int kSmLongQ = 16;                             // float4 per thread
-constexpr int kSmLongMax = kSmLongQ * 4 * kSmLongBlock - 8;  // (less what a misaligned start costs)
+constexpr int kSmLongQ = 16;                             // float4 per thread of the long-row kernel
+constexpr int kSmLongMax = kSmLongQ * 4 * kSmBlock - 8;  // (less what a misaligned start costs)
+constexpr int kSmByLane = 8, kSmBy8 = 96, kSmBy32 = 512, kSmByWave16 = 1024;  // row lengths up to which a lane / 8 lanes / 32 lanes / the wave with 16 entries per lane work on a row
 
 __device__ __forceinline__ int softmax_row_class(int64_t len) { return len <= kSmChunk ? 0 : len <= kSmLongMax ? 1 : 2; }
 
@@ -47,9 +46,9 @@ static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
 
 // First kernel: the layout, one thread per chunk (two binary searches of row_ptr whose loads the other
 // threads' searches hide).  With r the row that holds entry c * kSmChunk, chunk c begins at r's first
-// entry (r short), after r's last (r long: the long-row kernel owns it; the chunk may come out empty) or
-// at entry c * kSmChunk itself (r huge); it ends where chunk c + 1 would begin if that row were short
-// (so a long row that starts past the chunk's rows is left out) or at the multiple (huge).
+// entry (r short), after r's last (r long; the chunk may come out empty) or at entry c * kSmChunk itself
+// (r huge); it ends where chunk c + 1 would begin if that row were short (so a long row that starts
+// past the chunk's rows is left out) or at the multiple (huge).
 __global__ __launch_bounds__(256)
 void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows)
 {
@@ -108,42 +107,17 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
-// One row's piece buf[b, e) of a chunk: the lanes that work on it take it into registers (R entries
-// each, so that the LDS reads are all in flight together and the row is read and written once), maximum,
-// exp(x - max), sum; a whole row is normalised, a piece of a huge row is left as exp(x - max) with
-// (max, sum) in *rec.  Three forms, by how many lanes work on the row.
-
-// one lane (rows of a few entries: no lane exchanges at all)
-__device__ __forceinline__ void softmax_piece_by_lane(float *buf, int b, int e, bool whole, float2 *rec)
-{
-    constexpr int R = 8;
-    float v[R];
-#pragma unroll
-    for (int k = 0; k < R; ++k) v[k] = b + k < e ? buf[b + k] : -INFINITY;
-    float m = v[0];
-#pragma unroll
-    for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
-    float sum = 0.f;
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-        v[k] = b + k < e ? exp_nonpositive(v[k] - m) : 0.f;
-        sum += v[k];
-    }
-    const float f = whole ? 1.0f / sum : 1.0f;
-#pragma unroll
-    for (int k = 0; k < R; ++k) if (b + k < e) buf[b + k] = v[k] * f;
-    if (!whole) *rec = make_float2(m, sum);
-}
-
-// a group of GW lanes, up to GW * R entries (all lanes of the group call this with the same row; the lane
-// exchanges stay inside the group)
+// One whole row of len entries at xr / outr by a group of GW lanes (GW = 1: the lane alone), R entries
+// per lane, all of them requested before the first is used.  Every lane of the wave runs through this
+// (the lane exchanges must not sit under a branch); `mine` says whether the lane's group has a row.
 template <int GW, int R>
-__device__ __forceinline__ void softmax_piece_by_group(float *buf, int b, int e, bool whole, float2 *rec)
+__device__ __forceinline__ void softmax_row_by_group(const float *xr, float *outr, int len, bool mine)
 {
-    const int i0 = b + (threadIdx.x & (GW - 1));
+    const int gl = threadIdx.x & (GW - 1);
+    if (!mine) len = 0;
     float v[R];
 #pragma unroll
-    for (int k = 0; k < R; ++k) v[k] = i0 + k * GW < e ? buf[i0 + k * GW] : -INFINITY;
+    for (int k = 0; k < R; ++k) v[k] = gl + k * GW < len ? xr[gl + k * GW] : -INFINITY;
     float m = v[0];
 #pragma unroll
     for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
@@ -151,211 +125,122 @@ __device__ __forceinline__ void softmax_piece_by_group(float *buf, int b, int e,
     float sum = 0.f;
 #pragma unroll
     for (int k = 0; k < R; ++k) {
-        v[k] = i0 + k * GW < e ? exp_nonpositive(v[k] - m) : 0.f;
+        v[k] = gl + k * GW < len ? exp_nonpositive(v[k] - m) : 0.f;
         sum += v[k];
     }
     sum = group_sum<GW>(sum);
-    const float f = whole ? 1.0f / sum : 1.0f;
+    const float inv = 1.0f / sum;
 #pragma unroll
-    for (int k = 0; k < R; ++k) if (i0 + k * GW < e) buf[i0 + k * GW] = v[k] * f;
-    if (!whole && i0 == b) *rec = make_float2(m, sum);
+    for (int k = 0; k < R; ++k) if (gl + k * GW < len) outr[gl + k * GW] = v[k] * inv;
 }
 
-// the whole workgroup, up to kSmBlock * R entries (every thread calls this with the same row).
-// red: 2 x (waves per workgroup) floats of LDS
-template <int R>
-__device__ __forceinline__ void softmax_piece_by_workgroup(float *buf, float *red, int b, int e, bool whole, float2 *rec)
+// The same for a row too long for the registers of its group: a first walk, R entries per lane at a time,
+// keeps a running maximum and the sum of exponentials relative to it; a second walk (the row is in the
+// caches by then) writes exp(x - max) / sum.
+template <int GW, int R>
+__device__ __forceinline__ void softmax_row_in_two_walks(const float *xr, float *outr, int len)
 {
-    constexpr int NW = kSmBlock / 64;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int i0 = b + threadIdx.x;
-    float v[R];
+    const int gl = threadIdx.x & (GW - 1);
+    float m = -INFINITY, sum = 0.f;
+    for (int base = gl; base < len; base += GW * R) {
+        float v[R];
 #pragma unroll
-    for (int k = 0; k < R; ++k) v[k] = i0 + k * kSmBlock < e ? buf[i0 + k * kSmBlock] : -INFINITY;
-    float m = v[0];
+        for (int k = 0; k < R; ++k) v[k] = base + k * GW < len ? xr[base + k * GW] : -INFINITY;
+        float mn = m;
 #pragma unroll
-    for (int k = 1; k < R; ++k) m = fmaxf(m, v[k]);
-    m = group_max<64>(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
+        for (int k = 0; k < R; ++k) mn = fmaxf(mn, v[k]);
+        sum = m == -INFINITY ? 0.f : sum * exp_nonpositive(m - mn);
 #pragma unroll
-    for (int w = 0; w < NW; ++w) m = fmaxf(m, red[w]);
-    float sum = 0.f;
-#pragma unroll
-    for (int k = 0; k < R; ++k) {
-        v[k] = i0 + k * kSmBlock < e ? exp_nonpositive(v[k] - m) : 0.f;
-        sum += v[k];
+        for (int k = 0; k < R; ++k) sum += base + k * GW < len ? exp_nonpositive(v[k] - mn) : 0.f;
+        m = mn;
     }
-    sum = group_sum<64>(sum);
-    if (lane == 0) red[NW + wave] = sum;
-    __syncthreads();  // (also: everyone has read the maxima, so the next row may overwrite them)
-    sum = 0.f;
+    const float all = group_max<GW>(m);
+    sum = m == -INFINITY ? 0.f : sum * exp_nonpositive(m - all);
+    sum = group_sum<GW>(sum);
+    const float inv = 1.0f / sum;
+    for (int base = gl; base < len; base += GW * R) {
+        float v[R];
 #pragma unroll
-    for (int w = 0; w < NW; ++w) sum += red[NW + w];
-    const float f = whole ? 1.0f / sum : 1.0f;
+        for (int k = 0; k < R; ++k) v[k] = base + k * GW < len ? xr[base + k * GW] : -INFINITY;
 #pragma unroll
-    for (int k = 0; k < R; ++k) if (i0 + k * kSmBlock < e) buf[i0 + k * kSmBlock] = v[k] * f;
-    if (!whole && threadIdx.x == 0) *rec = make_float2(m, sum);
-    // (the sums are read before the next row's second barrier, which comes after its first: no barrier needed here)
+        for (int k = 0; k < R; ++k) if (base + k * GW < len) outr[base + k * GW] = exp_nonpositive(v[k] - all) * inv;
+    }
 }
 
-// piece lengths up to which a row is worked on by a lane / a group of 16 lanes / a wave; beyond: the workgroup
-constexpr int kSmByLane = 8, kSmBy16 = 192, kSmByWave = 1023;
-constexpr int kSmList16 = 2 * kSmChunk / (kSmByLane + 1) + 1, kSmList64 = 2 * kSmChunk / (kSmBy16 + 1) + 1,
-              kSmListWg = 2 * kSmChunk / (kSmByWave + 1) + 1;
-
-__global__ __launch_bounds__(kSmBlock, 3)  // (three waves per SIMD: 168 registers, a chunk ahead takes 36 of them)
-void sddmm_row_softmax_chunk_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                    float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
+// Second kernel: the short rows, a wave per chunk.
+__global__ __launch_bounds__(kSmBlock, 4)  // (at least four waves per SIMD; it takes 80 registers, so six fit)
+void sddmm_row_softmax_short_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                    const int4 *__restrict__ g_softmax_rows)
 {
-    __shared__ __align__(16) float buf[kSmBuf];
-    __shared__ int32_t rows_lds[kSmRowsMax];
-    __shared__ float red[2 * kSmBlock / 64];
-    // rows of the chunk that take more than a lane, by class (index of the row inside the round's window)
-    __shared__ uint16_t list16[kSmList16], list64[kSmList64], list_wg[kSmListWg];
-    __shared__ int n_listed[3];
-    constexpr int kPer = (kSmBuf / 4 + kSmBlock - 1) / kSmBlock;  // float4 per thread and chunk, at most
+    const int lane = threadIdx.x & 63;
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
-    // A chunk travels memory -> registers -> LDS as the float4 pieces from the aligned address below its
-    // first entry on; the registers are filled one chunk ahead, so the memory latency of chunk c + grid
-    // passes while chunk c is worked on.  The layout of a chunk says what to read, so the layouts are
-    // fetched two chunks ahead.
-    typedef float vec4 __attribute__((ext_vector_type(4)));  // (a plain vector: stays in registers through the conditional loads)
-    vec4 ahead[kPer];
-    auto layout_of = [&](int64_t c) { return c < n_chunks ? g_softmax_rows[c] : make_int4(0, 0, 0, 0); };
-    auto request = [&](int4 lay) __attribute__((always_inline)) {
-        if (vec_in && lay.x < lay.y) {
-            const int64_t a0 = lay.x & ~3;
-            const int nq = (int)((lay.y - a0 + 3) >> 2);
-            const vec4 *src = reinterpret_cast<const vec4 *>(x + a0);
-#pragma unroll
-            for (int u = 0; u < kPer; ++u) {
-                const int q = threadIdx.x + u * kSmBlock;
-                // (the last float4 of the array may reach beyond its end: that one is read entry by entry below)
-                if (q < nq && a0 + 4 * (int64_t)q + 3 < nnz) ahead[u] = src[q];
+    const int64_t n_waves = (int64_t)gridDim.x * (kSmBlock / 64);
+    for (int64_t c = (int64_t)blockIdx.x * (kSmBlock / 64) + (threadIdx.x >> 6); c < n_chunks; c += n_waves) {
+        const int4 lay = g_softmax_rows[c];
+        if (lay.x >= lay.y) continue;
+        for (int64_t w0 = lay.z; w0 <= lay.w; w0 += 64) {
+            const int64_t r = w0 + lane;
+            int64_t rb = 0;
+            int len = 0;
+            if (r <= lay.w) {
+                rb = row_ptr[r];
+                const int64_t l = (int64_t)row_ptr[r + 1] - rb;
+                len = l <= kSmChunk ? (int)l : 0;  // (a huge row at either end of the chunk is not this kernel's)
             }
-        }
-    };
-    int4 lay_cur = layout_of(blockIdx.x), lay_nxt = layout_of((int64_t)blockIdx.x + gridDim.x);
-    request(lay_cur);
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const int4 lay_after = layout_of(c + 2 * (int64_t)gridDim.x);
-        const int4 lay = lay_cur;
-        lay_cur = lay_nxt;
-        lay_nxt = lay_after;
-        if (lay.x >= lay.y) {  // no short or huge rows here
-            request(lay_cur);
-            continue;
-        }
-        const int64_t c0 = lay.x, c1 = lay.y;
-        const int64_t a0 = vec_in ? (c0 & ~(int64_t)3) : c0;  // buf[i] holds entry a0 + i
-        const int n = (int)(c1 - a0);
-        __syncthreads();  // the chunk before has left the buffers
-        if (vec_in) {
-            const int nq = (n + 3) >> 2;
+            // a lane per row
+            if (__ballot(len >= 1 && len <= kSmByLane)) softmax_row_by_group<1, kSmByLane>(x + rb, out + rb, len, len <= kSmByLane);
+            // groups of 8 lanes: eight rows at a time
+            uint64_t todo = __ballot(len > kSmByLane && len <= kSmBy8);
+            while (todo) {
+                int src = -1;  // the lane that holds the row of this lane's group
 #pragma unroll
-            for (int u = 0; u < kPer; ++u) {
-                const int q = threadIdx.x + u * kSmBlock;
-                if (q < nq) {
-                    if (a0 + 4 * (int64_t)q + 3 < nnz) {
-                        reinterpret_cast<vec4 *>(buf)[q] = ahead[u];
-                    } else {
-                        for (int j = 0; j < 4; ++j) buf[4 * q + j] = a0 + 4 * q + j < nnz ? x[a0 + 4 * q + j] : 0.f;
-                    }
+                for (int g = 0; g < 8; ++g) {
+                    const int b = todo ? __builtin_ctzll(todo) : -1;
+                    if (todo) todo &= todo - 1;
+                    if ((lane >> 3) == g) src = b;
                 }
+                const int64_t gb = __shfl(rb, src < 0 ? lane : src);
+                const int gn = __shfl(len, src < 0 ? lane : src);
+                softmax_row_by_group<8, kSmBy8 / 8>(x + gb, out + gb, gn, src >= 0);
             }
-        } else {
-            for (int i0 = threadIdx.x; i0 < n; i0 += 8 * kSmBlock) {
-                float v[8];
+            // groups of 32 lanes: two rows at a time
+            todo = __ballot(len > kSmBy8 && len <= kSmBy32);
+            while (todo) {
+                int src = -1;
 #pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = i0 + u * kSmBlock < n ? x[a0 + i0 + u * kSmBlock] : 0.f;
-#pragma unroll
-                for (int u = 0; u < 8; ++u) if (i0 + u * kSmBlock < n) buf[i0 + u * kSmBlock] = v[u];
-            }
-        }
-        const int64_t r0 = lay.z, r1 = lay.w;
-        // The chunk's row pointers go into LDS, kSmRowsMax - 1 rows at a time (one round unless the chunk is
-        // full of empty rows).  These loads are issued before the next chunk is requested, so that waiting
-        // for them does not wait for it.
-        for (int64_t w0 = r0; w0 <= r1; w0 += kSmRowsMax - 1) {
-            const int n_w = (int)(min(r1, w0 + kSmRowsMax - 2) - w0 + 1);  // rows of this round
-            if (w0 != r0) __syncthreads();  // the round before has left rows_lds and the lists
-            for (int i = threadIdx.x; i <= n_w; i += kSmBlock) rows_lds[i] = row_ptr[w0 + i];
-            if (threadIdx.x < 3) n_listed[threadIdx.x] = 0;
-            if (w0 == r0) request(lay_cur);
-            __syncthreads();
-            // (positions inside buf; only a huge row can reach beyond the chunk)
-            auto piece = [&](int k, int *b, int *e, bool *whole, float2 **rec) {
-                const int64_t rb = rows_lds[k], re = rows_lds[k + 1];
-                *b = (int)(max(rb, c0) - a0); *e = (int)(min(re, c1) - a0);
-                if (softmax_row_class(re - rb) == 1) *e = *b;  // (no long row lies inside a chunk; should one, it is left alone)
-                *whole = rb >= c0 && re <= c1;
-                *rec = &g_softmax_rec[2 * c + (rb < c0 ? 0 : 1)];
-            };
-            // every thread looks at the rows k = t, t + 256, ...: the short ones it does itself, the others it lists
-            for (int k = threadIdx.x; k < n_w; k += kSmBlock) {
-                int b, e; bool whole; float2 *rec;
-                piece(k, &b, &e, &whole, &rec);
-                const int len = e - b;
-                if (len <= 0) continue;
-                if (len <= kSmByLane) softmax_piece_by_lane(buf, b, e, whole, rec);
-                else if (len <= kSmBy16) list16[atomicAdd(&n_listed[0], 1)] = (uint16_t)k;
-                else if (len <= kSmByWave) list64[atomicAdd(&n_listed[1], 1)] = (uint16_t)k;
-                else list_wg[atomicAdd(&n_listed[2], 1)] = (uint16_t)k;
-            }
-            __syncthreads();
-            const int n16 = n_listed[0], n64 = n_listed[1], n_wg = n_listed[2];
-            for (int q = 0; q < n_wg; ++q) {
-                int b, e; bool whole; float2 *rec;
-                piece(list_wg[q], &b, &e, &whole, &rec);
-                if (e - b <= 8 * kSmBlock) softmax_piece_by_workgroup<8>(buf, red, b, e, whole, rec);
-                else softmax_piece_by_workgroup<kSmChunk / kSmBlock>(buf, red, b, e, whole, rec);
-            }
-            for (int q = threadIdx.x >> 6; q < n64; q += kSmBlock / 64) {
-                int b, e; bool whole; float2 *rec;
-                piece(list64[q], &b, &e, &whole, &rec);
-                if (e - b <= 6 * 64) softmax_piece_by_group<64, 6>(buf, b, e, whole, rec);
-                else softmax_piece_by_group<64, (kSmByWave + 63) / 64>(buf, b, e, whole, rec);
-            }
-            for (int q = threadIdx.x >> 4; q < n16; q += kSmBlock / 16) {
-                int b, e; bool whole; float2 *rec;
-                piece(list16[q], &b, &e, &whole, &rec);
-                if (e - b <= 4 * 16) softmax_piece_by_group<16, 4>(buf, b, e, whole, rec);
-                else softmax_piece_by_group<16, kSmBy16 / 16>(buf, b, e, whole, rec);
-            }
-        }
-        __syncthreads();
-        const int lo = (int)(c0 - a0);  // 0 .. 3: the entries before belong to the chunk or the long row before
-        if (vec_in && vec_out) {
-            float4 *dst = reinterpret_cast<float4 *>(out + a0);
-            const int nq = (n + 3) >> 2;
-#pragma unroll
-            for (int u = 0; u < kPer; ++u) {
-                const int q = threadIdx.x + u * kSmBlock, i = 4 * q;
-                if (q >= nq) continue;
-                if (i >= lo && i + 4 <= n) {
-                    dst[q] = reinterpret_cast<const float4 *>(buf)[q];
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) if (i + j >= lo && i + j < n) out[a0 + i + j] = buf[i + j];
+                for (int g = 0; g < 2; ++g) {
+                    const int b = todo ? __builtin_ctzll(todo) : -1;
+                    if (todo) todo &= todo - 1;
+                    if ((lane >> 5) == g) src = b;
                 }
+                const int64_t gb = __shfl(rb, src < 0 ? lane : src);
+                const int gn = __shfl(len, src < 0 ? lane : src);
+                softmax_row_by_group<32, kSmBy32 / 32>(x + gb, out + gb, gn, src >= 0);
             }
-        } else {
-            for (int i = lo + threadIdx.x; i < n; i += kSmBlock) out[a0 + i] = buf[i];
+            // the whole wave: row by row
+            todo = __ballot(len > kSmBy32);
+            while (todo) {
+                const int b = __builtin_ctzll(todo);
+                todo &= todo - 1;
+                const int64_t gb = __shfl(rb, b);
+                const int gn = __shfl(len, b);
+                if (gn <= kSmByWave16) softmax_row_by_group<64, kSmByWave16 / 64>(x + gb, out + gb, gn, true);
+                else softmax_row_in_two_walks<64, kSmByWave16 / 64>(x + gb, out + gb, gn);
+            }
         }
     }
 }
 
-// One long row [rb, re) by a workgroup of kSmLongBlock threads, the row held in registers (4 * NQ floats
-// per thread): read once, written once.  x 16-byte aligned: float4 pieces counted from the aligned
-// address below the row's start (entries outside the row are masked); otherwise single entries, strided.
+// One long row, or one piece of a huge row, [rb, re) by a workgroup of kSmBlock threads, held in registers
+// (4 * NQ floats per thread): read once, written once.  x 16-byte aligned: float4 pieces counted from the
+// aligned address below the first entry (entries outside are masked); otherwise single entries, strided.
+// rec = NULL: a whole row, normalised; otherwise a piece, stored as exp(x - max) with (max, sum) in *rec.
 template <int NQ>
 __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int64_t rb, int64_t re, int64_t nnz, bool vec_in,
-                                                 bool vec_out, float *red)
+                                                 bool vec_out, float *red, float2 *rec)
 {
-    constexpr int NW = kSmLongBlock / 64;
+    constexpr int NW = kSmBlock / 64;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     // (offsets relative to the aligned address below the row's start fit 32 bits)
     const int64_t a0 = vec_in ? (rb & ~(int64_t)3) : rb;
@@ -367,7 +252,7 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
     if (vec_in) {
 #pragma unroll
         for (int k = 0; k < NQ; ++k) {
-            const int p = 4 * (t + k * kSmLongBlock);
+            const int p = 4 * (t + k * kSmBlock);
             float4 v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
             if (p < end) {
                 if (p + 3 < lim) {
@@ -386,7 +271,7 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
     } else {
 #pragma unroll
         for (int k = 0; k < 4 * NQ; ++k) {
-            const int p = t + k * kSmLongBlock;
+            const int p = t + k * kSmBlock;
             f[k] = p < end ? xr[p] : -INFINITY;
         }
     }
@@ -410,11 +295,12 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
     sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += red[NW + w];
-    const float inv = 1.0f / sum;
+    const float inv = rec ? 1.0f : 1.0f / sum;
+    if (rec && t == 0) *rec = make_float2(m, sum);
     if (vec_in) {
 #pragma unroll
         for (int k = 0; k < NQ; ++k) {
-            const int p = 4 * (t + k * kSmLongBlock);
+            const int p = 4 * (t + k * kSmBlock);
             if (p >= end) continue;
             if (vec_out && p >= head && p + 4 <= end) {
                 *reinterpret_cast<float4 *>(outr + p) = make_float4(f[4 * k] * inv, f[4 * k + 1] * inv, f[4 * k + 2] * inv, f[4 * k + 3] * inv);
@@ -426,47 +312,62 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
     } else {
 #pragma unroll
         for (int k = 0; k < 4 * NQ; ++k) {
-            const int p = t + k * kSmLongBlock;
+            const int p = t + k * kSmBlock;
             if (p < end) outr[p] = f[k] * inv;
         }
     }
     // (the next row writes its maxima after this row's second barrier and its sums after its own first: no barrier needed here)
 }
 
-// The long rows.  A long row holds the multiple of kSmChunk that follows its first entry, so it is the
-// row after the last row of the chunk whose window [c * kSmChunk, (c + 1) * kSmChunk) it starts in.
-// Workgroup b looks at the chunks b, b + grid, ...: first at many of them at once, a thread per chunk
-// (three dependent loads each, which a walk chunk by chunk would pay for one after the other), the long
-// rows that start in them collected in a list; then the list row by row.
-__global__ __launch_bounds__(kSmLongBlock, 4)  // (four waves per SIMD = 128 registers: four rows in flight per compute unit)
+// Third kernel: the long rows and the pieces of huge rows.  A long row holds the multiple of kSmChunk
+// that follows its first entry, so it is the row after the last row of the chunk whose window
+// [c * kSmChunk, (c + 1) * kSmChunk) it starts in; a huge row is the first or the last row of every chunk
+// it touches.  Workgroup b looks at the chunks b, b + grid, ...: first at many of them at once, a thread
+// per chunk (a few dependent loads each, which a walk chunk by chunk would pay for one after the other),
+// what it finds collected in a list; then the list item by item.
+__global__ __launch_bounds__(kSmBlock, 4)  // (four waves per SIMD: four rows in flight per compute unit)
 void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                   const int4 *__restrict__ g_softmax_rows)
+                                   float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
 {
-    __shared__ float red[2 * kSmLongBlock / 64];
-    __shared__ int2 todo[kSmLongBlock];
+    __shared__ float red[2 * kSmBlock / 64];
+    __shared__ int4 todo[3 * kSmBlock];  // first entry, end, record (-1: a whole row)
     __shared__ int n_todo;
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
-    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmLongBlock) {
+    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmBlock) {
         __syncthreads();  // the list of the round before has been worked off
         if (threadIdx.x == 0) n_todo = 0;
         __syncthreads();
         const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
         if (c < n_chunks) {
-            const int64_t r = (int64_t)g_softmax_rows[c].w + 1;
+            const int4 lay = g_softmax_rows[c];
+            const int64_t r = (int64_t)lay.w + 1;
             if (r < n_rows) {
                 const int64_t rb = row_ptr[r], re = row_ptr[r + 1];
                 if (rb >= c * kSmChunk && rb < (c + 1) * kSmChunk && softmax_row_class(re - rb) == 1)
-                    todo[atomicAdd(&n_todo, 1)] = make_int2((int)rb, (int)re);
+                    todo[atomicAdd(&n_todo, 1)] = make_int4((int)rb, (int)re, -1, 0);
+            }
+            if (lay.x < lay.y) {
+                const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
+                const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1];
+                if (softmax_row_class(e0 - b0) == 2)
+                    todo[atomicAdd(&n_todo, 1)] = make_int4((int)max(b0, c0), (int)min(e0, c1), (int)(2 * c + (b0 < c0 ? 0 : 1)), 0);
+                if (r1 != r0) {
+                    const int64_t b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
+                    if (softmax_row_class(e1 - b1) == 2)
+                        todo[atomicAdd(&n_todo, 1)] = make_int4((int)max(b1, c0), (int)min(e1, c1), (int)(2 * c + 1), 0);
+                }
             }
         }
         __syncthreads();
         const int n = n_todo;
         for (int q = 0; q < n; ++q) {
-            const int64_t rb = todo[q].x, re = todo[q].y;
-            if (re - rb <= 8 * 4 * kSmLongBlock - 8) softmax_long_row<8>(x, out, rb, re, nnz, vec_in, vec_out, red);
-            else softmax_long_row<kSmLongQ>(x, out, rb, re, nnz, vec_in, vec_out, red);
+            const int4 w = todo[q];
+            const int64_t rb = w.x, re = w.y;
+            float2 *rec = w.z < 0 ? nullptr : &g_softmax_rec[w.z];
+            if (re - rb <= 8 * 4 * kSmBlock - 8) softmax_long_row<8>(x, out, rb, re, nnz, vec_in, vec_out, red, rec);
+            else softmax_long_row<kSmLongQ>(x, out, rb, re, nnz, vec_in, vec_out, red, rec);
         }
     }
 }
@@ -725,17 +626,15 @@ int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_
     } else if (int rc = softmax_store(&rec, &rows)) {
         return rc;
     }
-    // (the entry count lives on the device: the grid is sized for the machine, the kernels stride over the chunks)
+    // (the entry count lives on the device: the grids are sized for the machine, the kernels stride over the chunks)
     const unsigned grid = 256 * 4;
-    const unsigned grid_chunk = 256 * 3;  // (168 registers: three workgroups per compute unit)
     hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows);
-    hipLaunchKernelGGL(sddmm_row_softmax_chunk_kernel, dim3(grid_chunk), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+    hipLaunchKernelGGL(sddmm_row_softmax_short_kernel, dim3(4 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+                       (const int4 *)rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
                        rec, (const int4 *)rows);
     hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out,
                        (const float2 *)rec, (const int4 *)rows);
-    // (the long rows are touched by neither kernel above: this one could run anywhere after the first)
-    hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(2 * grid), dim3(kSmLongBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
-                       (const int4 *)rows);
     return last_error("sddmm_row_softmax");
 }
 

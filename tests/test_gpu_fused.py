@@ -41,12 +41,13 @@ def test_row_softmax_matches_oracle(oracle, cfg, scale):
 
 @pytest.mark.parametrize("misalign", [0, 1])
 def test_row_softmax_edge_rows(oracle, misalign):
-    """Rows at the boundaries of the kernel's cases: rows of up to 4096 entries are worked on in chunks of whole rows; inside
-    a chunk a row goes to a lane (up to 8 entries), 16 lanes (up to 192), a wave (up to 1023) or the workgroup; longer rows
-    have a kernel of their own (next test); a chunk's row pointers are staged 1151 rows at a time."""
-    lens = ([0, 1, 0, 8, 9, 64, 65, 192, 193, 1023, 1024, 0, 2, 511]      # every class, whole rows
-            + [4096 - sum([1, 8, 9, 64, 65, 192, 193, 1023, 1024, 2, 511])]  # ... up to the end of chunk 0 exactly
-            + [4096]                                                        # a row that is exactly chunk 1
+    """Rows at the boundaries of the kernel's cases: rows of up to 4096 entries are grouped into chunks of whole rows, a wave
+    takes a chunk 64 rows at a time and gives a row to a lane (up to 8 entries), 8 lanes (up to 96), 32 lanes (up to 512)
+    or all its lanes (up to 1024 in registers, beyond that in two walks); longer rows have a kernel of their own (next
+    test).  The runs of empty rows span several chunks' worth of row pointers."""
+    lens = ([0, 1, 0, 8, 9, 64, 65, 96, 97, 192, 193, 512, 513, 1023, 1024, 1025, 0, 2, 511]      # every class, whole rows
+            + [2 * 4096 - sum([1, 8, 9, 64, 65, 96, 97, 192, 193, 512, 513, 1023, 1024, 1025, 2, 511])]  # ... up to the end of chunk 1 exactly
+            + [4096]                                                        # a row that is exactly chunk 2
             + [5000, 3]                                                     # a row over two chunk boundaries, then a short one
             + [0] * 6000 + [1, 2] * 700 + [0] * 5000                        # runs of empty rows longer than a staging round
             + [13000]                                                       # a row over three boundaries with whole chunks inside
