@@ -113,8 +113,7 @@ def test_row_softmax_long_rows(oracle, misalign):
 
 
 @pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])
-def test_execute_softmax_matches_oracle(oracle, monkeypatch, kernel, K):
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
+def test_execute_softmax_matches_oracle(oracle, kernel, K):
     kid = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}[kernel]
     d = synth.make(3, 0.03, K=K, seed=12)
     d["W"] = d["W"] * 8.0; d["H"] = d["H"] * 8.0  # logits of order one
@@ -125,7 +124,8 @@ def test_execute_softmax_matches_oracle(oracle, monkeypatch, kernel, K):
     want = oracle.row_softmax(d["row_ptr"].numpy(), cpu_logits)
     # host-created plan (values inside) and device-created plan (values at execute)
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
-    plan = S.plan(K, 0, 0, kid)
+    opt = capi.PlanOptions.defaults(ignore_env=1, kernel=kid, split_min_nnz=0)
+    plan = S.plan(K, options=opt)
     plan.execute_softmax(0, W.data_ptr(), H.data_ptr(), out.data_ptr())
     torch.cuda.synchronize()
     got = out.cpu().numpy()
@@ -135,7 +135,7 @@ def test_execute_softmax_matches_oracle(oracle, monkeypatch, kernel, K):
     sums = np.bincount(d["row_ind"].numpy(), weights=got.astype(np.float64), minlength=d["n_rows"])
     assert np.allclose(sums[np.diff(d["row_ptr"].numpy()) > 0], 1.0, atol=1e-5)
     rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev); dv = d["val"].to(dev)
-    p2 = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, 0, 0, kid)
+    p2 = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, options=opt)
     out2 = torch.full_like(out, float("nan"))
     p2.execute_softmax(dv.data_ptr(), W.data_ptr(), H.data_ptr(), out2.data_ptr())
     torch.cuda.synchronize()

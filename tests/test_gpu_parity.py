@@ -16,13 +16,18 @@ KERNELS = {"row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": 
            "hybrid": capi.KERNEL_HYBRID, "auto": capi.KERNEL_AUTO}
 
 
-def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_vals=True):
-    """d: dict from synth (CPU tensors).  Returns (out numpy, plan info)."""
+def plan_options(kernel=capi.KERNEL_AUTO, tile_x=0, tile_y=0, **fields):
+    """The planner steered through sddmm_plan_options (the environment layer switched off)."""
+    return capi.PlanOptions.defaults(ignore_env=1, kernel=kernel, tile_size_x=tile_x, tile_size_y=tile_y, **fields)
+
+
+def run_gpu(d, K=None, tile_x=0, tile_y=0, kernel=capi.KERNEL_AUTO, use_plan_vals=True, opts=None):
+    """d: dict from synth (CPU tensors); opts: fields of sddmm_plan_options.  Returns (out numpy, plan info)."""
     dev = torch.device("cuda:0")
     rows = d["row_ind"].numpy(); cols = d["col_ind"].numpy(); vals = d["val"].numpy()
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], rows, cols, vals)
     K = K or d["K"]
-    plan = S.plan(K, tile_x, tile_y, kernel)
+    plan = S.plan(K, tile_x, tile_y, kernel) if opts is None else S.plan(K, options=plan_options(kernel, tile_x, tile_y, **opts))
     W = d["W"].to(dev).contiguous(); H = d["H"].to(dev).contiguous()
     out = torch.full((d["nnz"],), float("nan"), device=dev)
     dval = 0 if use_plan_vals else d["val"].to(dev)
@@ -134,13 +139,11 @@ def _dict_of(n, m, r, c, K, rng):
 
 
 @pytest.mark.parametrize("forced", [False, True])
-def test_extreme_shapes_through_the_planner(oracle, monkeypatch, forced):
+def test_extreme_shapes_through_the_planner(oracle, forced):
     """Degenerate shapes through AUTO and HYBRID, once with the planner's own choices
     and once with its size thresholds removed, so that the tiled and split plans (and
     their short batches) are built for inputs they would normally never see."""
-    if forced:
-        monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
-        monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")
+    opts = dict(split_min_nnz=0, stage_factor=0) if forced else None
     rng = np.random.default_rng(123)
     wide = np.unique(rng.integers(0, 150000, 60000))
     cases = [
@@ -160,7 +163,7 @@ def test_extreme_shapes_through_the_planner(oracle, monkeypatch, forced):
     for name, n, m, r, c, K in cases:
         d = _dict_of(n, m, r, c, K, rng)
         for kernel in ("auto", "hybrid"):
-            out, info = run_gpu(d, kernel=KERNELS[kernel])
+            out, info = run_gpu(d, kernel=KERNELS[kernel], opts=opts)
             rep = check(d, out, oracle)
             assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"], (name, kernel, info)
 
@@ -260,15 +263,14 @@ def residual_ok(out, d, oracle, K):
 
 @pytest.mark.parametrize("kernel,K", [("row", 32), ("row", 100), ("row", 30), ("lds", 64), ("lds", 100), ("panel", 128),
                                       ("panel", 512), ("auto", 32), ("auto", 64), ("auto", 128), ("auto", 256), ("auto", 512)])
-def test_residual_epilogue(oracle, monkeypatch, kernel, K):
+def test_residual_epilogue(oracle, kernel, K):
     """out = val - dot fused into every kernel family's store, with the values owned
     by the plan (stream order) and passed at execute (sorted order), in one K slice
     and in several; the scaled form through the same entry point gives sddmm_execute's bits."""
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
     d = synth.make(3, 0.05, K=K, seed=21)
     dev = torch.device("cuda:0")
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
-    plan = S.plan(K, 0, 0, KERNELS[kernel])
+    plan = S.plan(K, options=plan_options(KERNELS[kernel], split_min_nnz=0))
     W = d["W"].to(dev); H = d["H"].to(dev); dv = d["val"].to(dev)
     out = torch.full((d["nnz"],), float("nan"), device=dev)
     plan.execute_epilogue(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), capi.EPILOGUE_RESIDUAL)
@@ -301,16 +303,15 @@ def test_residual_epilogue_needs_values():
 
 
 @pytest.mark.parametrize("K", [64, 256])
-def test_execute_can_be_captured_in_a_graph(oracle, monkeypatch, K):
+def test_execute_can_be_captured_in_a_graph(oracle, K):
     """sddmm_execute only launches kernels on the caller's stream (no allocation, no
     memset, no synchronisation), so a caller may record it into a HIP graph.  The graph
     is replayed several times with eager work and synchronisations in between and with
     W changed in place; every replay must give the eager result's bits."""
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # the split plan: two launches per K slice
     d = synth.make(3, 0.05, K=K, seed=31)
     dev = torch.device("cuda:0")
     S = capi.Coo.from_arrays(d["n_rows"], d["n_cols"], d["row_ind"].numpy(), d["col_ind"].numpy(), d["val"].numpy())
-    plan = S.plan(K, 0, 0, capi.KERNEL_AUTO)
+    plan = S.plan(K, options=plan_options(split_min_nnz=0))  # the split plan: two launches per K slice
     W = d["W"].to(dev).contiguous(); H = d["H"].to(dev).contiguous()
     out = torch.zeros(d["nnz"], device=dev); eager = torch.zeros(d["nnz"], device=dev)
     side = torch.cuda.Stream()
@@ -361,15 +362,13 @@ def test_power_of_two_scaling_is_exact_and_tilings_agree(oracle):
 
 
 @pytest.mark.parametrize("short_max", [20, 100, 10 ** 9, 0])
-def test_hybrid_row_classes(oracle, monkeypatch, short_max):
+def test_hybrid_row_classes(oracle, short_max):
     """Forces the two row classes of a hybrid plan (long: tile kernel, short: padded
     gather) through the length threshold and checks the union of their outputs."""
-    monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(short_max))
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")  # split even this small matrix
-    monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")
     d = synth.make(3, 0.02, K=128)
     deg = np.diff(d["row_ptr"].numpy())
-    out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID)
+    # (split even this small matrix)
+    out, info = run_gpu(d, tile_x=100, kernel=capi.KERNEL_HYBRID, opts=dict(short_row_max=short_max, split_min_nnz=0, stage_factor=0))
     check(d, out, oracle)
     assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]
     assert sum(info["class_rows"]) == int((deg > 0).sum())
@@ -378,24 +377,22 @@ def test_hybrid_row_classes(oracle, monkeypatch, short_max):
         assert info["class_rows"][0] == int((deg >= 20).sum())
 
 
-@pytest.mark.parametrize("K,env", [
+@pytest.mark.parametrize("K,opts", [
     (64, {}), (192, {}), (256, {}), (512, {}),
-    (128, {"SDDMM_TILE_WAVES": "16"}),                      # 16 instead of 12 waves per workgroup
-    (128, {"SDDMM_TILE_ASSIGN": "1"}), (128, {"SDDMM_TILE_ASSIGN": "0"}),   # other work assignments
-    (256, {"SDDMM_TILE_KSLICE": "256"}),                    # one full-K slice: variant G=16, 4 float4 per lane
-    (512, {"SDDMM_TILE_KSLICE": "256", "SDDMM_DENSE": "0"}),                    # two slices of 256
-    (512, {"SDDMM_TILE_KSLICE": "512", "SDDMM_DENSE": "0"}),                    # variant G=16 or 32
-    (128, {"SDDMM_TILE_G": "4"}),                           # groups of 4 lanes in the tile kernel
-    (128, {"SDDMM_GATHER_G": "4"}), (256, {"SDDMM_GATHER_PADDED": "0"}),
+    (128, dict(tile_waves=16)),                             # 16 instead of 12 waves per workgroup
+    (128, dict(tile_assign=1)), (128, dict(tile_assign=0)),  # other work assignments
+    (256, dict(k_slice=256)),                               # one full-K slice: variant G=16, 4 float4 per lane
+    (512, dict(k_slice=256, dense_blocks=0)),               # two slices of 256
+    (512, dict(k_slice=512, dense_blocks=0)),               # variant G=16 or 32
+    (128, dict(tile_lanes=4)),                              # groups of 4 lanes in the tile kernel
+    (128, dict(gather_lanes=4)), (256, dict(gather_padded=0)),
 ])
-def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
+def test_hybrid_plan_ranks_and_variants(oracle, K, opts):
     """The split plan (tile kernel + padded gather) at several ranks and with the
-    planner's alternatives forced through their environment switches."""
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    planner's alternatives forced through the options."""
+    opts = dict(opts, split_min_nnz=0)
     d = synth.make(3, 0.06, K=K, seed=77)
-    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO, opts=opts)
     check(d, out, oracle)
     assert info["dense_nnz"] + sum(info["class_nnz"]) == d["nnz"]
     assert info["kernel"] == capi.KERNEL_HYBRID and info["class_nnz"][0] + info["dense_nnz"] > 0 and info["class_nnz"][2] > 0, info
@@ -403,7 +400,7 @@ def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
     dev = torch.device("cuda:0")
     dd = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
     plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], dd["row_ptr"].data_ptr(), dd["col_ind"].data_ptr(),
-                                     K, 0, 0, capi.KERNEL_AUTO)
+                                     K, options=plan_options(**opts))
     plan.set_values(dd["val"].data_ptr())
     out2 = torch.full((d["nnz"],), float("nan"), device=dev)
     plan.execute(0, dd["W"].data_ptr(), dd["H"].data_ptr(), out2.data_ptr())
@@ -411,31 +408,28 @@ def test_hybrid_plan_ranks_and_variants(oracle, monkeypatch, K, env):
     assert np.array_equal(out2.cpu().numpy(), out)
 
 
-@pytest.mark.parametrize("K,env", [(128, {}), (256, {}), (512, {}), (128, {"SDDMM_TILE_WAVES": "16"})])
-def test_short_batches(oracle, monkeypatch, K, env):
+@pytest.mark.parametrize("K,opts", [(128, {}), (256, {}), (512, {}), (128, dict(tile_waves=16))])
+def test_short_batches(oracle, K, opts):
     """Run ends with at most four nonzeros are collected, eight to a batch, into
     batches that the tile kernel runs in half the steps (both halves of a group of
     eight lanes then hold the same nonzeros).  The plan must report such batches, the
     results must stay within the tolerance of the oracle, two executes must give the
     same bits (the duplicate positions store the same value to the same place), and
     with the switch off there are none."""
-    monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    opts = dict(opts, split_min_nnz=0)
     d = synth.make(3, 0.06, K=K, seed=5)
-    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    out, info = run_gpu(d, kernel=capi.KERNEL_AUTO, opts=opts)
     check(d, out, oracle)
     assert info["short_batches"] > 0 and info["short_batches"] * 64 < info["padded_positions"], info
-    out_again, _ = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    out_again, _ = run_gpu(d, kernel=capi.KERNEL_AUTO, opts=opts)
     assert np.array_equal(out, out_again)
-    monkeypatch.setenv("SDDMM_TILE_SHORT", "0")
-    out_off, info_off = run_gpu(d, kernel=capi.KERNEL_AUTO)
+    out_off, info_off = run_gpu(d, kernel=capi.KERNEL_AUTO, opts=dict(opts, tile_short_batches=0))
     check(d, out_off, oracle)
     assert info_off["short_batches"] == 0 and info_off["padded_positions"] <= info["padded_positions"]
 
 
 @pytest.mark.parametrize("seed", list(range(48)))
-def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
+def test_random_shapes_kernels_and_tilings(oracle, seed):
     """Seeded random shapes, densities, ranks, kernels and tile sizes; every second
     case lets the planner split even a small matrix into its row classes."""
     rng = np.random.default_rng(1000 + seed)
@@ -443,11 +437,11 @@ def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
     K = int(rng.choice([4, 8, 12, 32, 64, 96, 128, 256, 512]))
     kernel = str(rng.choice(["auto", "row", "lds", "hybrid", "panel"]))
     tile_x = int(rng.choice([0, 1, 7, 64, 192, 320, 5000])); tile_y = int(rng.choice([0, 1, 33, 50000]))
+    opts = None
     if seed % 2:
-        monkeypatch.setenv("SDDMM_SPLIT_MIN_NNZ", "0")
-        monkeypatch.setenv("SDDMM_STAGE_FACTOR", "0")  # tile even where staging the H tiles does not pay
         rng.integers(2, 200)  # (keeps the random stream of the cases that follow)
-        monkeypatch.setenv("SDDMM_SHORT_ROW_MAX", str(int(rng.integers(1, 40))))
+        # (tile even where staging the H tiles does not pay)
+        opts = dict(split_min_nnz=0, stage_factor=0, short_row_max=int(rng.integers(1, 40)))
     # rows of very unequal length: a few long ones, many short or empty ones
     deg = np.minimum(n_cols, (rng.pareto(1.2, n_rows) * rng.integers(1, 30)).astype(np.int64))
     deg[rng.random(n_rows) < 0.2] = 0
@@ -462,7 +456,7 @@ def test_random_shapes_kernels_and_tilings(oracle, monkeypatch, seed):
              val=torch.from_numpy(rng.standard_normal(len(r)).astype(np.float32)),
              W=torch.from_numpy(rng.standard_normal((n_rows, K)).astype(np.float32)),
              H=torch.from_numpy(rng.standard_normal((n_cols, K)).astype(np.float32)))
-    out, info = run_gpu(d, tile_x=tile_x, tile_y=tile_y, kernel=KERNELS[kernel])
+    out, info = run_gpu(d, tile_x=tile_x, tile_y=tile_y, kernel=KERNELS[kernel], opts=opts)
     rows_np = d["row_ind"].numpy(); cols_np = d["col_ind"].numpy(); vals = d["val"].numpy()
     cpu = oracle.sddmm_csr(d["row_ptr"].numpy(), cols_np, vals, d["W"].numpy(), d["H"].numpy())
     _, absp = oracle.sddmm_f64(rows_np, cols_np, vals, d["W"].numpy(), d["H"].numpy())
