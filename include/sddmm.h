@@ -111,6 +111,18 @@ int sddmm_write_mtx(const sddmm_coo *S, const char *path);
 int sddmm_write_bin(const sddmm_coo *S, const char *path);
 int sddmm_read_bin(const char *path, sddmm_coo **out);
 
+/* A synthetic matrix of one of the five benchmark shapes, (row, col)-sorted:
+ * config 1 uniform 4096^2 at 1 %; 2 bag of words 1500 x 12,419 (lognormal row
+ * lengths, Zipf(1.1) columns, counts as values); 3 recommender 480,189 x 17,770
+ * (power-law row lengths, Zipf(0.9) columns, ratings 1..5; about 100 M nonzeros);
+ * 4 R-MAT 2^22 (200 M edges before duplicates are removed); 5 banded 2^20 (64 per
+ * row inside +-2048 of the diagonal).  scale in (0, 1] shrinks the dimensions
+ * (the nonzeros shrink with them); the result depends on (config, scale, seed)
+ * only, not on the number of host threads.  No counterpart in the reference,
+ * whose inputs are downloaded files (HiPC18/run.sh:3-6): this is what the
+ * command-line tool's --gen reads instead of a file.                          */
+int sddmm_coo_generate(int32_t config, double scale, uint64_t seed, sddmm_coo **out);
+
 /* Copies caller arrays (host) into a new matrix.  vals may be NULL (all 1). */
 int sddmm_coo_create(int64_t n_rows, int64_t n_cols, int64_t nnz, const int32_t *rows,
                      const int32_t *cols, const float *vals, sddmm_coo **out);

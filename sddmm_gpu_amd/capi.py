@@ -83,6 +83,7 @@ SIGNATURES = {
     "sddmm_write_mtx": (c_int, [c_void_p, c_char_p]),
     "sddmm_write_bin": (c_int, [c_void_p, c_char_p]),
     "sddmm_read_bin": (c_int, [c_char_p, POINTER(c_void_p)]),
+    "sddmm_coo_generate": (c_int, [c_int32, C.c_double, C.c_uint64, POINTER(c_void_p)]),
     "sddmm_coo_create": (c_int, [c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, POINTER(c_void_p)]),
     "sddmm_coo_destroy": (None, [c_void_p]),
     "sddmm_coo_info": (c_int, [c_void_p, POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int)]),
@@ -184,6 +185,13 @@ class Coo:
     def read_bin(cls, path):
         h = c_void_p()
         check(lib().sddmm_read_bin(str(path).encode(), byref(h)))
+        return cls(h)
+
+    @classmethod
+    def generate(cls, config, scale=1.0, seed=None):
+        """One of the five benchmark shapes, generated on the host (sddmm_coo_generate)."""
+        h = c_void_p()
+        check(lib().sddmm_coo_generate(config, float(scale), config if seed is None else seed, byref(h)))
         return cls(h)
 
     def write_mtx(self, path):

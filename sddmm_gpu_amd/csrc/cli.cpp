@@ -43,6 +43,9 @@ static void usage()
             "  --cpu-only     run the CPU path only (no GPU needed) and time it\n"
             "  --cpu-threads N  threads of the CPU path (default: all cores)\n"
             "  --seed N       srand48 seed of the dense factors (default 0, the reference's)\n"
+            "  --gen C[:S[:N]]  do not read `input`: generate benchmark shape C (1 uniform, 2 bag of words, 3 recommender,\n"
+            "                 4 R-MAT, 5 banded) at scale S in (0, 1] (default 1) with generator seed N (default: C);\n"
+            "                 `input` is then only a name -- with --save-bin the generated matrix is written out\n"
             "  --json         also print one JSON line with the plan and timing\n");
 }
 
@@ -79,7 +82,7 @@ int main(int argc, char **argv)
     bool plan_loaded = false;
     int runs = 1, cpu_threads = 0;
     long seed = 0;
-    std::string check_file, dump_file;
+    std::string check_file, dump_file, gen;
     uint32_t kernel = SDDMM_KERNEL_AUTO;
     std::string save_bin;
     for (int i = 5; i < argc; ++i) {
@@ -96,6 +99,7 @@ int main(int argc, char **argv)
         else if (a == "--seed" && i + 1 < argc) seed = atol(argv[++i]);
         else if (a == "--runs" && i + 1 < argc) runs = std::max(1, atoi(argv[++i]));
         else if (a == "--save-bin" && i + 1 < argc) save_bin = argv[++i];
+        else if (a == "--gen" && i + 1 < argc) gen = argv[++i];
         else if (a == "--kernel" && i + 1 < argc) {
             std::string k = argv[++i];
             if (k == "auto") kernel = SDDMM_KERNEL_AUTO;
@@ -110,7 +114,13 @@ int main(int argc, char **argv)
 
     auto t0 = std::chrono::steady_clock::now();
     sddmm_coo *S = nullptr;
-    if (ends_with(input, ".bin")) CHECK(sddmm_read_bin(input.c_str(), &S));
+    if (!gen.empty()) {
+        int config = 0; double scale = 1.0; unsigned long long gseed = 0;
+        const int got = sscanf(gen.c_str(), "%d:%lf:%llu", &config, &scale, &gseed);
+        if (got < 1) { fprintf(stderr, "sddmm: --gen takes CONFIG[:SCALE[:SEED]]\n"); return 2; }
+        if (got < 3) gseed = (unsigned long long)config;
+        CHECK(sddmm_coo_generate(config, scale, gseed, &S));
+    } else if (ends_with(input, ".bin")) CHECK(sddmm_read_bin(input.c_str(), &S));
     else CHECK(sddmm_read_mtx(input.c_str(), &S));
     int64_t n_rows, n_cols, nnz;
     int sorted;
@@ -163,7 +173,7 @@ int main(int argc, char **argv)
                    std::to_string(kernel) + ".plan";
         };
         // a plan file beside a binary input: built for this matrix, K and options, or ignored
-        if (plan_file && ends_with(input, ".bin")) {
+        if (plan_file && gen.empty() && ends_with(input, ".bin")) {
             if (sddmm_plan_load(plan_path(input).c_str(), S, (int32_t)K, &opt, &plan) == SDDMM_OK) plan_loaded = true;
             else plan = nullptr;
         }

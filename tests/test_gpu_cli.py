@@ -128,3 +128,17 @@ def test_cli_tile_size_y_shapes_the_row_ranges_of_a_wide_matrix(oracle, tmp_path
                        env=dict(os.environ, SDDMM_SPLIT_MIN_NNZ="0", SDDMM_TILE_FEW_BLOCKS="0"))
     assert r.returncode == 0, r.stderr + r.stdout
     assert "tile_size_Y = 64 is not used by this plan" in r.stderr, r.stderr
+
+
+def test_cli_on_a_generated_matrix():
+    """--gen: the tool makes the benchmark shape itself (no input file) and checks the device result per nonzero
+    against the library's CPU path."""
+    r = subprocess.run([CLI, "recommender", "128", "0", "0", "--gen", "3:0.02", "--check", "--json"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr + r.stdout
+    m = re.search(r"Matrix info:  rows: (\d+), cols: (\d+), nnz: (\d+)", r.stdout)
+    assert m and int(m.group(1)) == int(480189 * 0.02) and int(m.group(3)) > 100000
+    assert re.search(r"diff values in CPU and GPU: 0 ", r.stdout), r.stdout
+    r = subprocess.run([CLI, "x", "32", "0", "0", "--gen", "9"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "config must be 1..5" in r.stderr
+

@@ -325,6 +325,64 @@ def test_cli_cpu_only_matches_oracle_per_nonzero(tmp_path, oracle):
     assert p.returncode == 1
 
 
+def test_generated_benchmark_shapes(tmp_path, oracle):
+    """sddmm_coo_generate: the five benchmark shapes made on the host.  Sorted, inside the matrix, without duplicates,
+    the same for the same (config, scale, seed) whatever the number of threads, and with the statistics the shapes are
+    defined by; the command-line tool reads one in place of a file and its CPU path agrees with the oracle on it."""
+    import subprocess
+    want = {1: (1024, 1024, 10.24, None), 2: (375, 3104, 124.4, None), 3: (24009, 3973, 90.0, None), 4: (65536, 65536, 40.0, None),
+            5: (65536, 65536, 62.6, 64)}
+    scale = {1: 0.25, 2: 0.25, 3: 0.05, 4: 2.0 ** -6, 5: 2.0 ** -4}
+    for cfg in range(1, 6):
+        S = capi.Coo.generate(cfg, scale[cfg], seed=7)
+        n_rows, n_cols, nnz, is_sorted = S.info()
+        r, c, v = S.arrays()
+        assert (n_rows, n_cols) == want[cfg][:2] and is_sorted and len(r) == nnz
+        key = r.astype(np.int64) * n_cols + c
+        assert np.all(np.diff(key) > 0) and r.min() >= 0 and r.max() < n_rows and c.min() >= 0 and c.max() < n_cols
+        deg = np.bincount(r, minlength=n_rows)
+        assert abs(deg.mean() / want[cfg][2] - 1) < 0.2, (cfg, deg.mean())
+        if want[cfg][3]:
+            assert deg.max() <= want[cfg][3]
+        assert np.all(np.isfinite(v)) and v.min() > 0
+        os.environ["SDDMM_NUM_THREADS"] = "1"
+        try:
+            r1, c1, v1 = capi.Coo.generate(cfg, scale[cfg], seed=7).arrays()
+        finally:
+            del os.environ["SDDMM_NUM_THREADS"]
+        assert np.array_equal(r, r1) and np.array_equal(c, c1) and np.array_equal(v, v1)
+        r2, c2, _ = capi.Coo.generate(cfg, scale[cfg], seed=8).arrays()
+        assert len(r2) != len(r) or not np.array_equal(c, c2)
+    # what defines the shapes: the band; the heavy tails of the recommender's rows and columns; R-MAT's hubs
+    r, c, v = capi.Coo.generate(5, 2.0 ** -4).arrays()
+    assert np.abs(c.astype(np.int64) - r).max() <= 2048 and np.abs(c.astype(np.int64) - r).max() > 1900
+    r, c, v = capi.Coo.generate(3, 0.05).arrays()
+    deg = np.sort(np.bincount(r))[::-1]; pop = np.sort(np.bincount(c))[::-1]
+    assert deg[: len(deg) // 100].sum() > 0.15 * len(r) and pop[: len(pop) // 10].sum() > 0.3 * len(c)
+    assert set(np.unique(v)) == {1.0, 2.0, 3.0, 4.0, 5.0}
+    r, c, v = capi.Coo.generate(4, 2.0 ** -6).arrays()
+    assert np.bincount(r).max() > 100 * (len(r) / 65536) and np.all(v == 1.0)
+    for bad in ((0, 1.0), (6, 1.0), (1, 0.0), (1, 1.5)):
+        with pytest.raises(capi.SddmmError) as e:
+            capi.Coo.generate(*bad)
+        assert e.value.code == capi.ERR_ARG
+    # the command-line tool on a generated matrix, CPU path, against the oracle's vector for the same matrix
+    cli = os.path.join(ROOT, "sddmm_gpu_amd", "bin", "sddmm")
+    S = capi.Coo.generate(2, 0.25)
+    n_rows, n_cols, nnz, _ = S.info()
+    r, c, v = S.arrays()
+    K = 16
+    vec = tmp_path / "want.f32"
+    oracle.sddmm_csr(S.row_ptr(), c, v, oracle.initial(n_rows, K), oracle.initial(n_cols, K)).tofile(vec)
+    p = subprocess.run([cli, "generated", str(K), "0", "0", "--gen", "2:0.25", "--cpu-only", "--check-against", str(vec),
+                        "--save-bin", str(tmp_path / "g.bin")], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr + p.stdout
+    assert "Matrix info:  rows: %d, cols: %d, nnz: %d" % (n_rows, n_cols, nnz) in p.stdout
+    assert "diff values in CPU and GPU: 0 " in p.stdout
+    r3, c3, v3 = capi.Coo.read_bin(tmp_path / "g.bin").arrays()
+    assert np.array_equal(r, r3) and np.array_equal(c, c3) and np.array_equal(v, v3)
+
+
 def test_sddmm_cpu_errors():
     S = capi.Coo.from_arrays(3, 3, [2, 0], [0, 1])  # unsorted
     with pytest.raises(capi.SddmmError) as e:
