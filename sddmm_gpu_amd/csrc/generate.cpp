@@ -172,16 +172,19 @@ extern "C" int sddmm_coo_generate(int32_t config, double scale, uint64_t seed, s
             const int sc = scale < 1.0 ? std::max(4, 22 + (int)std::lround(std::log2(scale))) : 22;
             const int64_t n = (int64_t)1 << sc, n_edges = std::max<int64_t>(16, (int64_t)(200e6 * scale));
             std::vector<uint64_t> keys((size_t)n_edges);
-            parallel_ranges(n_edges, 1 << 16, [&](int64_t b, int64_t e, int) {
-                Rng g(seed, (uint64_t)b);
-                for (int64_t i = b; i < e; ++i) {
-                    uint64_t row = 0, col = 0;
-                    for (int l = 0; l < sc; ++l) {
-                        const double u = g.uniform();
-                        row = row * 2 + (u >= 0.76);
-                        col = col * 2 + ((u >= 0.57 && u < 0.76) || u >= 0.95);
+            constexpr int64_t kBlock = 4096;  // edges per generator, so that the result does not depend on where the threads' ranges begin
+            parallel_ranges((n_edges + kBlock - 1) / kBlock, 16, [&](int64_t b, int64_t e, int) {
+                for (int64_t blk = b; blk < e; ++blk) {
+                    Rng g(seed, (uint64_t)blk);
+                    for (int64_t i = blk * kBlock; i < std::min(n_edges, (blk + 1) * kBlock); ++i) {
+                        uint64_t row = 0, col = 0;
+                        for (int l = 0; l < sc; ++l) {
+                            const double u = g.uniform();
+                            row = row * 2 + (u >= 0.76);
+                            col = col * 2 + ((u >= 0.57 && u < 0.76) || u >= 0.95);
+                        }
+                        keys[(size_t)i] = row << 32 | col;
                     }
-                    keys[(size_t)i] = row << 32 | col;
                 }
             });
             std::sort(keys.begin(), keys.end());

@@ -330,6 +330,7 @@ def test_generated_benchmark_shapes(tmp_path, oracle):
     the same for the same (config, scale, seed) whatever the number of threads, and with the statistics the shapes are
     defined by; the command-line tool reads one in place of a file and its CPU path agrees with the oracle on it."""
     import subprocess
+    cli = os.path.join(ROOT, "sddmm_gpu_amd", "bin", "sddmm")
     want = {1: (1024, 1024, 10.24, None), 2: (375, 3104, 124.4, None), 3: (24009, 3973, 90.0, None), 4: (65536, 65536, 40.0, None),
             5: (65536, 65536, 62.6, 64)}
     scale = {1: 0.25, 2: 0.25, 3: 0.05, 4: 2.0 ** -6, 5: 2.0 ** -4}
@@ -345,11 +346,12 @@ def test_generated_benchmark_shapes(tmp_path, oracle):
         if want[cfg][3]:
             assert deg.max() <= want[cfg][3]
         assert np.all(np.isfinite(v)) and v.min() > 0
-        os.environ["SDDMM_NUM_THREADS"] = "1"
-        try:
-            r1, c1, v1 = capi.Coo.generate(cfg, scale[cfg], seed=7).arrays()
-        finally:
-            del os.environ["SDDMM_NUM_THREADS"]
+        # (the thread count is read once per process: the one-thread run is the command-line tool's)
+        one = tmp_path / ("one%d.bin" % cfg)
+        p = subprocess.run([cli, "x", "4", "0", "0", "--gen", "%d:%r:7" % (cfg, scale[cfg]), "--cpu-only", "--save-bin", str(one)],
+                           capture_output=True, text=True, timeout=120, env=dict(os.environ, SDDMM_NUM_THREADS="1"))
+        assert p.returncode == 0, p.stderr + p.stdout
+        r1, c1, v1 = capi.Coo.read_bin(one).arrays()
         assert np.array_equal(r, r1) and np.array_equal(c, c1) and np.array_equal(v, v1)
         r2, c2, _ = capi.Coo.generate(cfg, scale[cfg], seed=8).arrays()
         assert len(r2) != len(r) or not np.array_equal(c, c2)
@@ -367,7 +369,6 @@ def test_generated_benchmark_shapes(tmp_path, oracle):
             capi.Coo.generate(*bad)
         assert e.value.code == capi.ERR_ARG
     # the command-line tool on a generated matrix, CPU path, against the oracle's vector for the same matrix
-    cli = os.path.join(ROOT, "sddmm_gpu_amd", "bin", "sddmm")
     S = capi.Coo.generate(2, 0.25)
     n_rows, n_cols, nnz, _ = S.info()
     r, c, v = S.arrays()
