@@ -12,6 +12,7 @@
 // bundle's runs are about equally long.  Rows too short for the tiles gather their H rows from
 // global memory, one group of lanes per row.
 #include <hip/hip_runtime.h>
+#include <utility>
 #include "kernels.hpp"
 
 using namespace sddmm;
@@ -19,6 +20,17 @@ using namespace sddmm;
 namespace {
 
 typedef float vec4f __attribute__((ext_vector_type(4)));
+
+// The value that lane I of this lane's group of 8 holds, by two row broadcasts of the data-parallel
+// primitives (one per half of a 16-lane row) and a select: vector-ALU work with no trip through the LDS
+// pipe, which the H reads keep busy and whose latency would sit in front of every round.
+template <int I>
+__device__ __forceinline__ int from_group_lane(int v, bool upper_group)
+{
+    const int lo = __builtin_amdgcn_update_dpp(0, v, 0x150 + I, 0xf, 0xf, false);      // row_newbcast:I
+    const int up = __builtin_amdgcn_update_dpp(0, v, 0x150 + I + 8, 0xf, 0xf, false);  // row_newbcast:I+8
+    return upper_group ? up : lo;
+}
 
 // KPL float4 per lane: a K slice of 32 * KPL elements on groups of 8 lanes
 template <int KPL, int NW>
@@ -63,7 +75,7 @@ void sddmm_spmm_tile_kernel(const SpmmArgs a)
         // A wave takes the bundles wave, wave + NW, ... of the item.  While bundle b is walked, the headers of bundle
         // b + 2 NW and the first three rounds of bundle b + NW are requested; inside a bundle round r + 3 is requested
         // while round r is computed.  A round is 8 steps: lane l of a group fetches the column and the value of the
-        // group's step 8 r + l, and the group's lanes take them from each other step by step.
+        // group's step 8 r + l, and the group's lanes take them from each other (from_group_lane).
         if (wi.begin + wave >= wi.end) continue;
         struct Hdr { int p0, len, off, n8; };
         auto header = [&](int b) -> Hdr {
@@ -100,15 +112,14 @@ void sddmm_spmm_tile_kernel(const SpmmArgs a)
             for (int r = 0; r < n8; ++r) {
                 const Round q3 = fetch(h0, r + 3);
                 // the columns (as row offsets in the tile) and the values of the round's eight steps, taken from the
-                // group's lanes (exchanging those of round r + 1 here instead measured 3 % slower)
+                // group's lanes
                 int row_off[8];
                 float xs[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int src = (lane & ~7) + i;
-                    row_off[i] = __shfl((int)q0.c, src) * (K4 * 16);
-                    xs[i] = __shfl(q0.x, src);
-                }
+                const int my_off = (int)q0.c * (K4 * 16), my_x = __float_as_int(q0.x);
+                const bool upper = (lane & 8) != 0;
+                [&]<int... I>(std::integer_sequence<int, I...>) {
+                    ((row_off[I] = from_group_lane<I>(my_off, upper), xs[I] = __int_as_float(from_group_lane<I>(my_x, upper))), ...);
+                }(std::make_integer_sequence<int, 8>{});
                 // the H pieces of step i + 1 are requested before the arithmetic of step i
                 vec4f hb[2][KPL];
                 rd(hb[0], row_off[0]);
