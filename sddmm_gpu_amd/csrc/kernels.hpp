@@ -1,4 +1,4 @@
-// Argument blocks and lookup functions shared by the plan builder (engine.hip)
+// Argument blocks and lookup functions shared by the plan builder (planner.hip, planner_tile.hip), the launch code (engine.hip)
 // and the kernel translation units.
 #pragma once
 #include <cstdint>
