@@ -344,6 +344,16 @@ def main():
         _, sm_ms, _ = time_steps(lambda st: capi.row_softmax(d["n_rows"], rp, x.data_ptr(), y.data_ptr(), st), n_steps, n_warm, torch, 30.0)
         _, es_ms, _ = time_steps(lambda st: plan.execute_softmax(0, d["W"].data_ptr(), d["H"].data_ptr(), y.data_ptr(), st),
                                  n_steps, n_warm, torch, 30.0)
+        # the softmax of the full-size result against the same thing written with torch's segment operations
+        torch.cuda.synchronize()
+        ri = d["row_ind"].to(torch.int64)
+        mx = torch.full((d["n_rows"],), float("-inf"), device=dev).scatter_reduce_(0, ri, x, "amax")
+        ref = torch.exp(x - mx[ri])
+        ref /= torch.zeros(d["n_rows"], device=dev).index_add_(0, ri, ref)[ri]
+        sm_diff = float(((y - ref).abs() / ref.clamp_min(1e-37)).max())
+        row_sums = torch.zeros(d["n_rows"], device=dev, dtype=torch.float64).index_add_(0, ri, y.double())
+        sm_sum_dev = float((row_sums[row_sums > 0] - 1.0).abs().max())
+        del ri, mx, ref, row_sums
         Y = torch.empty(d["n_rows"], K0, device=dev)
         _, sp_ms, _ = time_steps(lambda st: capi.spmm_csr(d["n_rows"], d["n_cols"], d["nnz"], rp, ci, y.data_ptr(), K0,
                                                           d["H"].data_ptr(), Y.data_ptr(), st), n_steps, n_warm, torch, 30.0)
@@ -362,7 +372,8 @@ def main():
         sp_bytes = 8.0 * d["nnz"] + 4.0 * (d["n_rows"] + 1) + 4.0 * K0 * (info["cols_touched"] + d["n_rows"])
         line["fused"] = {
             "row_softmax": {"ms": round(sm_ms, 4), "alg_bytes": sm_bytes, "alg_gbps": round(sm_bytes / (sm_ms * 1e6), 1),
-                            "hbm_frac": round(sm_bytes / (sm_ms * 1e6) / HBM_PEAK_GBPS, 4)},
+                            "hbm_frac": round(sm_bytes / (sm_ms * 1e6) / HBM_PEAK_GBPS, 4),
+                            "max_rel_diff_vs_torch": sm_diff, "max_row_sum_minus_one": sm_sum_dev},
             "sddmm_plus_softmax": {"ms": round(es_ms, 4)},
             "spmm_csr": {"ms": round(sp_ms, 4), "gflops": round(2.0 * d["nnz"] * K0 / (sp_ms * 1e6), 1), "alg_bytes": sp_bytes,
                          "alg_gbps": round(sp_bytes / (sp_ms * 1e6), 1), "hbm_frac": round(sp_bytes / (sp_ms * 1e6) / HBM_PEAK_GBPS, 4)},
