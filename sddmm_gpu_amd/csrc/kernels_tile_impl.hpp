@@ -314,6 +314,12 @@ void sddmm_tile_kernel(const TileArgs a)
     constexpr bool XORDER = !GATHER && (K4 % 16 == 0);
     constexpr bool COMPACT = !GATHER && K4 <= 16;  // the compact stream format (see TileArgs)
     constexpr bool STREAM_HINT = !GATHER && !COMPACT && SLICE == 0;  // (see ld_meta)
+    // The compact stream serves the thin K slices, where a batch is little arithmetic and the kernel moves
+    // at the rate of its requests in flight: 16 waves x 2 batches x 448 bytes of index data per compute unit
+    // are 14 KB, and at a microsecond of memory latency 256 compute units then fetch 3.6 TB/s -- what the
+    // K = 32 launch measured.  Its index data is therefore requested four batches ahead (the arrays' slack
+    // of 256 entries covers exactly the four batches past the end).
+    constexpr bool DEEP = COMPACT;
     constexpr int ROW_SHIFT = K4 == 16 ? 8 : K4 == 8 ? 7 : 0;  // log2 of an LDS row in bytes (COMPACT only)
     // SHORTS: a batch may be marked "short" in a.btype: each of its groups then holds at most G/2
     // nonzeros in its first G/2 positions and the same ones again in the other G/2.  With the
@@ -637,30 +643,37 @@ void sddmm_tile_kernel(const TileArgs a)
         if (b0 < bf) {
             Meta m0 = issue_meta();
             Meta m1 = issue_meta();
+            // DEEP: the index data is requested four batches ahead instead of two (see DEEP)
+            Meta d2, d3;
+            if constexpr (DEEP) { d2 = issue_meta(); d3 = issue_meta(); }
             issue_old(m0);
             issue_w(wa, m0.wrow);
             columns_of_steps<G, XORDER>(m0.col, lane_base0, ca);
-            Meta m2 = issue_meta();
+            Meta m2 = DEEP ? d2 : issue_meta();
+            Meta m3 = DEEP ? d3 : Meta{};
+            Meta m4 = DEEP ? issue_meta() : Meta{};
             issue_old(m1);
             issue_w(wb, m1.wrow);
             __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the arithmetic
             run(b0, wa, m0, ca, cb, m1.col);
             for (int bi = b0 + 1; bi < bf; bi += 2) {
                 flush();
-                Meta m3 = issue_meta();
+                const Meta n0 = issue_meta();  // batch bi + 2 (DEEP: bi + 4)
+                if constexpr (!DEEP) m3 = n0;
                 issue_old(m2);
                 issue_w(wa, m2.wrow);
                 __builtin_amdgcn_sched_barrier(0);
                 run(bi, wb, m1, cb, ca, m2.col);
                 if (bi + 1 >= bf) break;
                 flush();
-                Meta m4 = issue_meta();
+                const Meta n1 = issue_meta();  // batch bi + 3 (DEEP: bi + 5)
                 issue_old(m3);
                 issue_w(wb, m3.wrow);
                 __builtin_amdgcn_sched_barrier(0);
                 run(bi + 1, wa, m2, ca, cb, m3.col);
                 m1 = m3;
-                m2 = m4;
+                if constexpr (DEEP) { m2 = m4; m3 = n0; m4 = n1; }
+                else m2 = n1;
             }
             flush();
         }
