@@ -336,3 +336,52 @@ def test_concurrent_executes_with_caller_workspaces(oracle, K, softmax):
     plan.execute_ws(0, W.data_ptr(), H.data_ptr(), out.data_ptr(), wss[0].data_ptr(), nbytes, capi.EPILOGUE_RESIDUAL)
     torch.cuda.synchronize()
     residual_ok(out.cpu().numpy(), d, oracle, K)
+
+
+def test_workspace_entry_points_reject_bad_arguments():
+    """sddmm_execute_ws and sddmm_plan_spmm check what they are given before anything is launched: a workspace that is
+    missing, too small or not 256-byte aligned, unknown bits in `form`, the residual form without values, NULL arrays."""
+    K = 256
+    d = synth.make(3, 0.03, K=K, seed=13)
+    dev = torch.device(DEV)
+    rp = d["row_ptr"].to(dev); ci = d["col_ind"].to(dev)
+    opt = capi.PlanOptions.defaults(ignore_env=1, split_min_nnz=0, stage_factor=0, spmm_stream=1)
+    plan = capi.Plan.from_device_csr(d["n_rows"], d["n_cols"], d["nnz"], rp.data_ptr(), ci.data_ptr(), K, options=opt)  # no values
+    nbytes = plan.workspace_bytes()
+    assert nbytes > 0 and plan.info()["k_slice"] < K
+    W = d["W"].to(dev); H = d["H"].to(dev); val = d["val"].to(dev)
+    out = torch.full((d["nnz"],), float("nan"), device=dev)
+    ws = torch.empty(nbytes + 512, dtype=torch.uint8, device=dev)
+    base = ws.data_ptr() + (-ws.data_ptr()) % 256
+    args = (val.data_ptr(), W.data_ptr(), H.data_ptr(), out.data_ptr())
+
+    def refused(call):
+        with pytest.raises(capi.SddmmError) as e:
+            call()
+        assert e.value.code == capi.ERR_ARG, e.value
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(out).all())  # nothing ran
+
+    refused(lambda: plan.execute_ws(*args, 0, 0))                                   # no workspace
+    refused(lambda: plan.execute_ws(*args, base, nbytes - 1))                       # too small
+    refused(lambda: plan.execute_ws(*args, base + 16, nbytes))                      # misaligned
+    refused(lambda: plan.execute_ws(*args, base, nbytes, 0x200))                    # unknown form bits
+    refused(lambda: plan.execute_ws(*args, base, nbytes, 7))                        # unknown epilogue
+    refused(lambda: plan.execute_ws(0, *args[1:], base, nbytes, capi.EPILOGUE_RESIDUAL))  # val - dot without values
+    refused(lambda: plan.execute_ws(args[0], 0, args[2], args[3], base, nbytes))    # NULL W
+    Y = torch.full((d["n_rows"], K), float("nan"), device=dev)
+    x = torch.ones(d["nnz"], device=dev)
+    for call in (lambda: plan.spmm(x.data_ptr(), H.data_ptr(), Y.data_ptr(), base, nbytes - 1),
+                 lambda: plan.spmm(x.data_ptr(), H.data_ptr(), Y.data_ptr(), base + 16, nbytes),
+                 lambda: plan.spmm(0, H.data_ptr(), Y.data_ptr()),
+                 lambda: plan.spmm(x.data_ptr(), H.data_ptr(), 0)):
+        with pytest.raises(capi.SddmmError) as e:
+            call()
+        assert e.value.code == capi.ERR_ARG, e.value
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(Y).all())
+    # and the good call still works afterwards
+    plan.execute_ws(*args, base, nbytes)
+    plan.spmm(x.data_ptr(), H.data_ptr(), Y.data_ptr(), base, nbytes)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(Y).all())
