@@ -384,7 +384,7 @@ int sddmm_execute_ws(const sddmm_plan *plan, const float *d_val, const float *d_
  * workgroup, by its length -- so it is read once and written once; a longer row
  * is cut into pieces of 4096 entries whose (max, sum) records are merged by a
  * last kernel.  The layout of the work and those records are kept in fixed
- * device arrays of the library (16 MiB per GPU), so softmax calls that overlap
+ * device arrays of the library (18 MiB per GPU), so softmax calls that overlap
  * in time on one GPU (different streams or threads) race unless they bring a
  * workspace (sddmm_execute_ws); calls on one stream never do.
  * sddmm_row_softmax: the same pass on its own, over any CSR pattern in device

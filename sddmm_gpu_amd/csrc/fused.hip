@@ -32,17 +32,20 @@ constexpr int kSmBlock = 256;
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
 constexpr int kSmLongQ = 16;                             // float4 per thread of the long-row kernel
 constexpr int kSmLongMax = kSmLongQ * 4 * kSmBlock - 8;  // (less what a misaligned start costs)
+constexpr int kSmOwnBatches = 32;                       // batches of 64 rows that a chunk's own wave takes at least
 constexpr int kSmByLane = 8, kSmBy8 = 96, kSmBy32 = 512, kSmByWave16 = 1024;  // row lengths up to which a lane / 8 lanes / 32 lanes / the wave with 16 entries per lane work on a row
 
 __device__ __forceinline__ int softmax_row_class(int64_t len) { return len <= kSmChunk ? 0 : len <= kSmLongMax ? 1 : 2; }
 
 // (m, sum) of the pieces of huge rows: [2c] the row that began before chunk c, [2c + 1] the row that ends
 // after it; and the layout of each chunk: first entry, end, first row, last row.  The kernels take both
-// arrays as arguments: a caller's workspace (sddmm_execute_ws), or these file-scope arrays, 8 + 8 MiB per
+// arrays as arguments: a caller's workspace (sddmm_execute_ws), or these file-scope arrays, 8 + 8 + 2 MiB per
 // device, held until the process ends -- softmax calls without a workspace that overlap in time on one
 // device share them and must not (calls on one stream never do).
 static __device__ __align__(256) float2 g_softmax_rec_store[2 * kSmMaxChunks];
 static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
+// [0]: how many chunks hold more rows than their own wave takes; from [1] on: those chunks (2 MiB more)
+static __device__ __align__(256) int32_t g_softmax_list_store[kSmMaxChunks + 64];
 
 // First kernel: the layout, one thread per chunk (two binary searches of row_ptr whose loads the other
 // threads' searches hide).  With r the row that holds entry c * kSmChunk, chunk c begins at r's first
@@ -50,8 +53,10 @@ static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
 // (r huge); it ends where chunk c + 1 would begin if that row were short (so a long row that starts
 // past the chunk's rows is left out) or at the multiple (huge).
 __global__ __launch_bounds__(256)
-void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows)
+void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows,
+                                   int32_t *__restrict__ g_softmax_list)
 {
+    if (blockIdx.x == 0 && threadIdx.x == 0) g_softmax_list[0] = 0;  // (the third kernel counts in it)
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * blockDim.x) {
@@ -167,23 +172,24 @@ __device__ __forceinline__ void softmax_row_in_two_walks(const float *xr, float 
     }
 }
 
-// Second kernel: the short rows, a wave per chunk.
-__global__ __launch_bounds__(kSmBlock, 4)  // (at least four waves per SIMD; it takes 80 registers, so six fit)
-void sddmm_row_softmax_short_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                    const int4 *__restrict__ g_softmax_rows)
+// How many batches of 64 rows the wave of a chunk takes itself.  A chunk with more rows than that (4096
+// entries spread over many rows: mostly empty ones) would hold its wave long after the others are done:
+// its further batches go to the whole machine (the last kernel), so no wave takes much more than twice the
+// average.
+__device__ __forceinline__ int64_t softmax_own_batches(int64_t n_rows, int64_t n_chunks)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t nnz = row_ptr[n_rows];
-    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    const int64_t n_waves = (int64_t)gridDim.x * (kSmBlock / 64);
-    for (int64_t c = (int64_t)blockIdx.x * (kSmBlock / 64) + (threadIdx.x >> 6); c < n_chunks; c += n_waves) {
-        const int4 lay = g_softmax_rows[c];
-        if (lay.x >= lay.y) continue;
-        for (int64_t w0 = lay.z; w0 <= lay.w; w0 += 64) {
+    return max((int64_t)kSmOwnBatches, 2 * (n_rows / (64 * max(n_chunks, (int64_t)1)) + 1));
+}
+
+// The short rows among the 64 rows from w0 (up to row `last`), by one wave.
+__device__ __forceinline__ void softmax_row_batch(const int32_t *__restrict__ row_ptr, const float *x, float *out, int64_t w0,
+                                                  int64_t last, int lane)
+{
+        {
             const int64_t r = w0 + lane;
             int64_t rb = 0;
             int len = 0;
-            if (r <= lay.w) {
+            if (r <= last) {
                 rb = row_ptr[r];
                 const int64_t l = (int64_t)row_ptr[r + 1] - rb;
                 len = l <= kSmChunk ? (int)l : 0;  // (a huge row at either end of the chunk is not this kernel's)
@@ -229,6 +235,23 @@ void sddmm_row_softmax_short_kernel(const int32_t *__restrict__ row_ptr, int64_t
                 else softmax_row_in_two_walks<64, kSmByWave16 / 64>(x + gb, out + gb, gn);
             }
         }
+}
+
+// Second kernel: the short rows, a wave per chunk.
+__global__ __launch_bounds__(kSmBlock, 4)  // (at least four waves per SIMD; it takes 80 registers, so six fit)
+void sddmm_row_softmax_short_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                    const int4 *__restrict__ g_softmax_rows)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t nnz = row_ptr[n_rows];
+    const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    const int64_t n_waves = (int64_t)gridDim.x * (kSmBlock / 64);
+    const int64_t own = softmax_own_batches(n_rows, n_chunks);
+    for (int64_t c = (int64_t)blockIdx.x * (kSmBlock / 64) + (threadIdx.x >> 6); c < n_chunks; c += n_waves) {
+        const int4 lay = g_softmax_rows[c];
+        if (lay.x >= lay.y) continue;
+        const int64_t last = min((int64_t)lay.w, (int64_t)lay.z + 64 * own - 1);
+        for (int64_t w0 = lay.z; w0 <= last; w0 += 64) softmax_row_batch(row_ptr, x, out, w0, last, lane);
     }
 }
 
@@ -327,7 +350,7 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
 // what it finds collected in a list; then the list item by item.
 __global__ __launch_bounds__(kSmBlock, 4)  // (four waves per SIMD: four rows in flight per compute unit)
 void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                   float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
+                                   float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows, int32_t *g_softmax_list)
 {
     __shared__ float red[2 * kSmBlock / 64];
     __shared__ int4 todo[3 * kSmBlock];  // first entry, end, record (-1: a whole row)
@@ -335,6 +358,7 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
+    const int64_t own = softmax_own_batches(n_rows, n_chunks);
     for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmBlock) {
         __syncthreads();  // the list of the round before has been worked off
         if (threadIdx.x == 0) n_todo = 0;
@@ -350,6 +374,8 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
             }
             if (lay.x < lay.y) {
                 const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
+                // (more rows than the chunk's own wave takes: the last kernel takes the others)
+                if ((r1 - r0) / 64 + 1 > own) g_softmax_list[1 + atomicAdd(&g_softmax_list[0], 1)] = (int32_t)c;
                 const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1];
                 if (softmax_row_class(e0 - b0) == 2)
                     todo[atomicAdd(&n_todo, 1)] = make_int4((int)max(b0, c0), (int)min(e0, c1), (int)(2 * c + (b0 < c0 ? 0 : 1)), 0);
@@ -409,15 +435,59 @@ __device__ __forceinline__ void scale_range(float *out, int64_t b, int64_t e, fl
     }
 }
 
-// Last kernel: the pieces of huge rows are scaled to the whole row's maximum and sum.  A chunk holds at
-// most two of them: at its beginning (the row came from the chunk before, or fills this one and goes on)
-// and at its end.
+// The batches of rows that the listed chunks' own waves left, spread over all workgroups: a chunk's further
+// batches in parts of kSmPart (one or two per wave of a workgroup), part p of list item i with the
+// workgroup (i + p) mod gridDim.x.  Every workgroup looks at the whole list, kSmBlock items at a time.
+constexpr int kSmPart = 2 * (kSmBlock / 64);
+__device__ __forceinline__ void softmax_rest_of_listed_chunks(const int32_t *__restrict__ row_ptr, int64_t n_rows, int64_t n_chunks,
+                                                              const float *x, float *out, const int4 *__restrict__ g_softmax_rows,
+                                                              const int32_t *__restrict__ g_softmax_list)
+{
+    __shared__ int64_t part_first[kSmBlock];  // first row of a list item's first part for this workgroup
+    __shared__ int part_last[kSmBlock];       // the item's last row
+    __shared__ int n_parts;
+    const int n_list = g_softmax_list[0];
+    if (n_list <= 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t own = softmax_own_batches(n_rows, n_chunks), G = gridDim.x;
+    for (int base = 0; base < n_list; base += kSmBlock) {
+        __syncthreads();
+        if (threadIdx.x == 0) n_parts = 0;
+        __syncthreads();
+        const int i = base + (int)threadIdx.x;
+        if (i < n_list) {
+            const int4 lay = g_softmax_rows[g_softmax_list[1 + i]];
+            const int64_t first = (int64_t)lay.z + 64 * own;  // (<= lay.w: that is why the chunk is listed)
+            const int64_t parts = (((int64_t)lay.w - first) / 64 + kSmPart) / kSmPart;
+            const int64_t p0 = (((int64_t)blockIdx.x - i) % G + G) % G;
+            if (p0 < parts) {
+                const int k = atomicAdd(&n_parts, 1);
+                part_first[k] = first + p0 * kSmPart * 64;
+                part_last[k] = lay.w;
+            }
+        }
+        __syncthreads();
+        const int n = n_parts;
+        for (int q = 0; q < n; ++q) {
+            const int64_t last = part_last[q];
+            for (int64_t p = part_first[q]; p <= last; p += G * kSmPart * 64)
+                for (int64_t w0 = p + 64 * wave; w0 <= min(last, p + kSmPart * 64 - 1); w0 += kSmBlock)
+                    softmax_row_batch(row_ptr, x, out, w0, last, lane);
+        }
+    }
+}
+
+// Last kernel.  First the rest of the short rows (above).  Then the pieces of huge rows are scaled to the
+// whole row's maximum and sum.  A chunk holds at most two of them: at its beginning (the row came from the
+// chunk before, or fills this one and goes on) and at its end.
 __global__ __launch_bounds__(kSmBlock)
-void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, float *out,
-                                    const float2 *__restrict__ g_softmax_rec, const int4 *__restrict__ g_softmax_rows)
+void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                    const float2 *__restrict__ g_softmax_rec, const int4 *__restrict__ g_softmax_rows,
+                                    const int32_t *__restrict__ g_softmax_list)
 {
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
+    softmax_rest_of_listed_chunks(row_ptr, n_rows, n_chunks, x, out, g_softmax_rows, g_softmax_list);
     // (like the long-row kernel: the chunks are looked at many at a time, the few with work listed)
     __shared__ int todo[kSmBlock];
     __shared__ int n_todo;
@@ -585,33 +655,37 @@ int last_error(const char *who)
 namespace sddmm {
 
 // device addresses of the file-scope record arrays on the current device (looked up once per device)
-static int softmax_store(float2 **rec, int4 **rows)
+static int softmax_store(float2 **rec, int4 **rows, int32_t **list)
 {
     constexpr int kMaxDevices = 64;
     static std::mutex mu;
     static float2 *rec_of[kMaxDevices] = {};
     static int4 *rows_of[kMaxDevices] = {};
+    static int32_t *list_of[kMaxDevices] = {};
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: no usable current device");
     std::lock_guard<std::mutex> lock(mu);
     if (!rec_of[dev]) {
-        void *a = nullptr, *b = nullptr;
+        void *a = nullptr, *b = nullptr, *c = nullptr;
         if ((e = hipGetSymbolAddress(&a, HIP_SYMBOL(g_softmax_rec_store))) != hipSuccess ||
-            (e = hipGetSymbolAddress(&b, HIP_SYMBOL(g_softmax_rows_store))) != hipSuccess || !a || !b)
+            (e = hipGetSymbolAddress(&b, HIP_SYMBOL(g_softmax_rows_store))) != hipSuccess ||
+            (e = hipGetSymbolAddress(&c, HIP_SYMBOL(g_softmax_list_store))) != hipSuccess || !a || !b || !c)
             return fail(SDDMM_ERR_HIP, "sddmm_row_softmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
         rec_of[dev] = static_cast<float2 *>(a);
         rows_of[dev] = static_cast<int4 *>(b);
+        list_of[dev] = static_cast<int32_t *>(c);
     }
     *rec = rec_of[dev];
     *rows = rows_of[dev];
+    *list = list_of[dev];
     return SDDMM_OK;
 }
 
 int64_t row_softmax_workspace_bytes(int64_t nnz)
 {
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    return ((n_chunks * 32 + 255) / 256) * 256;  // two float2 and one int4 per chunk
+    return (((n_chunks * 36 + 4) + 255) / 256) * 256;  // two float2, one int4 and one list item per chunk, and the list's count
 }
 
 int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream, void *d_ws, int64_t nnz)
@@ -619,22 +693,24 @@ int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_
     if (n_rows <= 0) return SDDMM_OK;
     float2 *rec = nullptr;
     int4 *rows = nullptr;
-    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] chunk layouts
+    int32_t *list = nullptr;
+    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] chunk layouts, then the list: its count and [n_chunks] items
         const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
         rec = static_cast<float2 *>(d_ws);
         rows = reinterpret_cast<int4 *>(rec + 2 * n_chunks);
-    } else if (int rc = softmax_store(&rec, &rows)) {
+        list = reinterpret_cast<int32_t *>(rows + n_chunks);
+    } else if (int rc = softmax_store(&rec, &rows, &list)) {
         return rc;
     }
     // (the entry count lives on the device: the grids are sized for the machine, the kernels stride over the chunks)
     const unsigned grid = 256 * 4;
-    hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows);
+    hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows, list);
     hipLaunchKernelGGL(sddmm_row_softmax_short_kernel, dim3(4 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
                        (const int4 *)rows);
     hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
-                       rec, (const int4 *)rows);
-    hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_out,
-                       (const float2 *)rec, (const int4 *)rows);
+                       rec, (const int4 *)rows, list);
+    hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x,
+                       d_out, (const float2 *)rec, (const int4 *)rows, (const int32_t *)list);
     return last_error("sddmm_row_softmax");
 }
 

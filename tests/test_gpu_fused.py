@@ -112,6 +112,27 @@ def test_row_softmax_long_rows(oracle, misalign):
     assert bool(torch.isnan(other[:3 - misalign]).all()) and bool(torch.isnan(other[3 - misalign + len(x):]).all())
 
 
+def test_row_softmax_mostly_empty_rows(oracle):
+    """A chunk of 4096 entries that spans far more rows than the average chunk (mostly empty rows) is not left to its own
+    wave: that wave takes twice the average number of rows (at least 2048), the rest is dealt out to all workgroups in
+    parts of 512 rows.  Here: ordinary rows, then 2.6 million rows with one to three entries in every 997th (more parts
+    than there are workgroups, so some take two), then ordinary rows again, a second such stretch with rows of every
+    short class in it, and the array ends inside a stretch of empty rows."""
+    rng = np.random.default_rng(5)
+    sparse = np.zeros(2_600_000, dtype=np.int64); sparse[::997] = rng.integers(1, 4, len(sparse[::997]))
+    second = np.zeros(400_000, dtype=np.int64); second[::15011] = np.resize([1, 8, 9, 96, 97, 512, 513, 1100], len(second[::15011]))
+    lens = np.concatenate([rng.integers(50, 150, 3000), sparse, rng.integers(0, 300, 2000), second, [7], np.zeros(70_000, dtype=np.int64)])
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    x = rng.normal(0, 5, rp[-1]).astype(np.float32)
+    dev = torch.device(DEV)
+    xd = torch.from_numpy(x).to(dev); out = torch.full_like(xd, float("nan")); rpd = torch.from_numpy(rp).to(dev)
+    for _ in range(2):  # (the second call finds the first one's list in the library's arrays)
+        out.fill_(float("nan"))
+        capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+        softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
+
+
 @pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])
 def test_execute_softmax_matches_oracle(oracle, kernel, K):
     kid = {"auto": capi.KERNEL_AUTO, "row": capi.KERNEL_ROW_GATHER, "lds": capi.KERNEL_LDS_TILE, "panel": capi.KERNEL_PANEL}[kernel]
