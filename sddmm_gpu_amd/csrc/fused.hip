@@ -32,6 +32,7 @@ constexpr int kSmBlock = 256;
 constexpr int64_t kSmMaxChunks = ((int64_t)1 << 31) / kSmChunk;
 constexpr int kSmLongQ = 16;                             // float4 per thread of the long-row kernel
 constexpr int kSmLongMax = kSmLongQ * 4 * kSmBlock - 8;  // (less what a misaligned start costs)
+constexpr int kSmListRows = 1 << 30, kSmListHuge = 1 << 29, kSmListChunk = kSmListHuge - 1;  // an item of the last kernel's list: flags | chunk
 constexpr int kSmOwnBatches = 32;                       // batches of 64 rows that a chunk's own wave takes at least
 constexpr int kSmByLane = 8, kSmBy8 = 96, kSmBy32 = 512, kSmByWave16 = 1024;  // row lengths up to which a lane / 8 lanes / 32 lanes / the wave with 16 entries per lane work on a row
 
@@ -44,7 +45,8 @@ __device__ __forceinline__ int softmax_row_class(int64_t len) { return len <= kS
 // device share them and must not (calls on one stream never do).
 static __device__ __align__(256) float2 g_softmax_rec_store[2 * kSmMaxChunks];
 static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
-// [0]: how many chunks hold more rows than their own wave takes; from [1] on: those chunks (2 MiB more)
+// the last kernel's work, 2 MiB: [0] and [1] the lengths of two lists of chunks (with flags), one from [2] upwards, the
+// other from [n_chunks + 1] downwards (a chunk is in one of them at most)
 static __device__ __align__(256) int32_t g_softmax_list_store[kSmMaxChunks + 64];
 
 // First kernel: the layout, one thread per chunk (two binary searches of row_ptr whose loads the other
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256)
 void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows,
                                    int32_t *__restrict__ g_softmax_list)
 {
-    if (blockIdx.x == 0 && threadIdx.x == 0) g_softmax_list[0] = 0;  // (the third kernel counts in it)
+    if (blockIdx.x == 0 && threadIdx.x < 2) g_softmax_list[threadIdx.x] = 0;  // (the third kernel counts in them)
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * blockDim.x) {
@@ -364,6 +366,7 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
         if (threadIdx.x == 0) n_todo = 0;
         __syncthreads();
         const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
+        int item = 0;  // this chunk's item of the last kernel's lists, if it has one
         if (c < n_chunks) {
             const int4 lay = g_softmax_rows[c];
             const int64_t r = (int64_t)lay.w + 1;
@@ -374,16 +377,41 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
             }
             if (lay.x < lay.y) {
                 const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
-                // (more rows than the chunk's own wave takes: the last kernel takes the others)
-                if ((r1 - r0) / 64 + 1 > own) g_softmax_list[1 + atomicAdd(&g_softmax_list[0], 1)] = (int32_t)c;
+                // for the last kernel: more rows than the chunk's own wave takes; pieces of huge rows
+                item = (r1 - r0) / 64 + 1 > own ? kSmListRows : 0;
                 const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1];
-                if (softmax_row_class(e0 - b0) == 2)
+                if (softmax_row_class(e0 - b0) == 2) {
                     todo[atomicAdd(&n_todo, 1)] = make_int4((int)max(b0, c0), (int)min(e0, c1), (int)(2 * c + (b0 < c0 ? 0 : 1)), 0);
+                    item |= kSmListHuge;
+                }
                 if (r1 != r0) {
                     const int64_t b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
-                    if (softmax_row_class(e1 - b1) == 2)
+                    if (softmax_row_class(e1 - b1) == 2) {
                         todo[atomicAdd(&n_todo, 1)] = make_int4((int)max(b1, c0), (int)min(e1, c1), (int)(2 * c + 1), 0);
+                        item |= kSmListHuge;
+                    }
                 }
+            }
+        }
+        // Chunks with rows left go to the list that all workgroups will read, chunks with pieces of huge rows
+        // only to the one of which a workgroup reads its share; one addition to a list's length per wave.
+        {
+            const int lane = threadIdx.x & 63;
+            const bool rows_left = item & kSmListRows;
+            const uint64_t front = __ballot(rows_left), back = __ballot(item && !rows_left), below = ((uint64_t)1 << lane) - 1;
+            if (front) {
+                const int first = __builtin_ctzll(front);
+                int at = 0;
+                if (lane == first) at = atomicAdd(&g_softmax_list[0], __builtin_popcountll(front));
+                at = __shfl(at, first);
+                if (rows_left) g_softmax_list[2 + at + __builtin_popcountll(front & below)] = item | (int)c;
+            }
+            if (back) {
+                const int first = __builtin_ctzll(back);
+                int at = 0;
+                if (lane == first) at = atomicAdd(&g_softmax_list[1], __builtin_popcountll(back));
+                at = __shfl(at, first);
+                if (item && !rows_left) g_softmax_list[n_chunks + 1 - at - __builtin_popcountll(back & below)] = item | (int)c;
             }
         }
         __syncthreads();
@@ -435,100 +463,85 @@ __device__ __forceinline__ void scale_range(float *out, int64_t b, int64_t e, fl
     }
 }
 
-// The batches of rows that the listed chunks' own waves left, spread over all workgroups: a chunk's further
-// batches in parts of kSmPart (one or two per wave of a workgroup), part p of list item i with the
-// workgroup (i + p) mod gridDim.x.  Every workgroup looks at the whole list, kSmBlock items at a time.
-constexpr int kSmPart = 2 * (kSmBlock / 64);
-__device__ __forceinline__ void softmax_rest_of_listed_chunks(const int32_t *__restrict__ row_ptr, int64_t n_rows, int64_t n_chunks,
-                                                              const float *x, float *out, const int4 *__restrict__ g_softmax_rows,
-                                                              const int32_t *__restrict__ g_softmax_list)
+// The pieces of huge rows in chunk c are scaled to the whole row's maximum and sum, by a workgroup.  A chunk
+// holds at most two of them: at its beginning (the row came from the chunk before, or fills this one and
+// goes on) and at its end.
+__device__ __forceinline__ void softmax_merge_chunk(const int32_t *__restrict__ row_ptr, float *out, const float2 *__restrict__ g_softmax_rec,
+                                                    const int4 *__restrict__ g_softmax_rows, int64_t c)
 {
-    __shared__ int64_t part_first[kSmBlock];  // first row of a list item's first part for this workgroup
-    __shared__ int part_last[kSmBlock];       // the item's last row
-    __shared__ int n_parts;
-    const int n_list = g_softmax_list[0];
-    if (n_list <= 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t own = softmax_own_batches(n_rows, n_chunks), G = gridDim.x;
-    for (int base = 0; base < n_list; base += kSmBlock) {
-        __syncthreads();
-        if (threadIdx.x == 0) n_parts = 0;
-        __syncthreads();
-        const int i = base + (int)threadIdx.x;
-        if (i < n_list) {
-            const int4 lay = g_softmax_rows[g_softmax_list[1 + i]];
-            const int64_t first = (int64_t)lay.z + 64 * own;  // (<= lay.w: that is why the chunk is listed)
-            const int64_t parts = (((int64_t)lay.w - first) / 64 + kSmPart) / kSmPart;
-            const int64_t p0 = (((int64_t)blockIdx.x - i) % G + G) % G;
-            if (p0 < parts) {
-                const int k = atomicAdd(&n_parts, 1);
-                part_first[k] = first + p0 * kSmPart * 64;
-                part_last[k] = lay.w;
-            }
-        }
-        __syncthreads();
-        const int n = n_parts;
-        for (int q = 0; q < n; ++q) {
-            const int64_t last = part_last[q];
-            for (int64_t p = part_first[q]; p <= last; p += G * kSmPart * 64)
-                for (int64_t w0 = p + 64 * wave; w0 <= min(last, p + kSmPart * 64 - 1); w0 += kSmBlock)
-                    softmax_row_batch(row_ptr, x, out, w0, last, lane);
-        }
+    const int4 lay = g_softmax_rows[c];
+    const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
+    const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
+    if (softmax_row_class(e0 - b0) == 2 && (b0 < c0 || e0 > c1)) {  // a huge row begins the chunk
+        const float2 all = merged_record(g_softmax_rec, b0, e0);
+        const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
+        const float f = expf(mine.x - all.x) / all.y;
+        const int64_t pb = max(b0, c0), pe = min(e0, c1);
+        scale_range(out, pb, pe, f);
+    }
+    if (r1 != r0 && softmax_row_class(e1 - b1) == 2 && e1 > c1) {  // another one begins inside the chunk and ends after it
+        const float2 all = merged_record(g_softmax_rec, b1, e1);
+        const float2 mine = g_softmax_rec[2 * c + 1];
+        const float f = expf(mine.x - all.x) / all.y;
+        scale_range(out, b1, c1, f);
     }
 }
 
-// Last kernel.  First the rest of the short rows (above).  Then the pieces of huge rows are scaled to the
-// whole row's maximum and sum.  A chunk holds at most two of them: at its beginning (the row came from the
-// chunk before, or fills this one and goes on) and at its end.
+// Last kernel, over the two lists that the third kernel made.
+//  - The chunks whose own wave left batches of rows.  Every workgroup reads that whole list, kSmBlock items
+//    at a time (on most matrices it is empty), and takes its share: a chunk's further batches in parts of
+//    kSmPart (one or two per wave of a workgroup), part p of list item i with the workgroup (i + p) mod
+//    gridDim.x; if the chunk holds pieces of huge rows too, workgroup i mod gridDim.x merges them.
+//  - The other chunks with pieces of huge rows: item i with the workgroup i mod gridDim.x.
+constexpr int kSmPart = 2 * (kSmBlock / 64);
+
 __global__ __launch_bounds__(kSmBlock)
 void sddmm_row_softmax_merge_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
                                     const float2 *__restrict__ g_softmax_rec, const int4 *__restrict__ g_softmax_rows,
                                     const int32_t *__restrict__ g_softmax_list)
 {
+    __shared__ int64_t todo_first[2 * kSmBlock];  // first row of this workgroup's first part of a chunk; or -1 - chunk: its huge rows' pieces
+    __shared__ int todo_last[2 * kSmBlock];       // the chunk's last row
+    __shared__ int n_todo;
+    const int n_list = g_softmax_list[0], n_huge = g_softmax_list[1];
+    if (n_list <= 0 && n_huge <= 0) return;
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    softmax_rest_of_listed_chunks(row_ptr, n_rows, n_chunks, x, out, g_softmax_rows, g_softmax_list);
-    // (like the long-row kernel: the chunks are looked at many at a time, the few with work listed)
-    __shared__ int todo[kSmBlock];
-    __shared__ int n_todo;
-    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmBlock) {
-        __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t own = softmax_own_batches(n_rows, n_chunks), G = gridDim.x;
+    for (int base = 0; base < n_list; base += kSmBlock) {
+        __syncthreads();  // the list of the round before has been worked off
         if (threadIdx.x == 0) n_todo = 0;
         __syncthreads();
-        {
-            const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
-            if (c < n_chunks) {
-                const int4 lay = g_softmax_rows[c];
-                if (lay.x < lay.y) {
-                    const int64_t r0 = lay.z, r1 = lay.w;
-                    if (softmax_row_class((int64_t)row_ptr[r0 + 1] - row_ptr[r0]) == 2 ||
-                        softmax_row_class((int64_t)row_ptr[r1 + 1] - row_ptr[r1]) == 2)
-                        todo[atomicAdd(&n_todo, 1)] = threadIdx.x;
-                }
+        const int i = base + (int)threadIdx.x;
+        if (i < n_list) {
+            const int item = g_softmax_list[2 + i], c = item & kSmListChunk;
+            const int4 lay = g_softmax_rows[c];
+            const int64_t first = (int64_t)lay.z + 64 * own;  // (<= lay.w: that is why the chunk is in this list)
+            const int64_t parts = (((int64_t)lay.w - first) / 64 + kSmPart) / kSmPart;
+            const int64_t p0 = (((int64_t)blockIdx.x - i) % G + G) % G;
+            if (p0 < parts) {
+                const int k = atomicAdd(&n_todo, 1);
+                todo_first[k] = first + p0 * kSmPart * 64;
+                todo_last[k] = lay.w;
             }
+            if ((item & kSmListHuge) && i % G == blockIdx.x) todo_first[atomicAdd(&n_todo, 1)] = -1 - (int64_t)c;
         }
         __syncthreads();
         const int n = n_todo;
         for (int q = 0; q < n; ++q) {
-            const int64_t c = base + (int64_t)todo[q] * gridDim.x;
-            const int4 lay = g_softmax_rows[c];
-            const int64_t c0 = lay.x, c1 = lay.y, r0 = lay.z, r1 = lay.w;
-            const int64_t b0 = row_ptr[r0], e0 = row_ptr[r0 + 1], b1 = row_ptr[r1], e1 = row_ptr[r1 + 1];
-            if (softmax_row_class(e0 - b0) == 2 && (b0 < c0 || e0 > c1)) {  // a huge row begins the chunk
-                const float2 all = merged_record(g_softmax_rec, b0, e0);
-                const float2 mine = g_softmax_rec[2 * c + (b0 < c0 ? 0 : 1)];
-                const float f = expf(mine.x - all.x) / all.y;
-                const int64_t pb = max(b0, c0), pe = min(e0, c1);
-                scale_range(out, pb, pe, f);
+            if (todo_first[q] < 0) {
+                softmax_merge_chunk(row_ptr, out, g_softmax_rec, g_softmax_rows, -1 - todo_first[q]);
+                continue;
             }
-            if (r1 != r0 && softmax_row_class(e1 - b1) == 2 && e1 > c1) {  // another one begins inside the chunk and ends after it
-                const float2 all = merged_record(g_softmax_rec, b1, e1);
-                const float2 mine = g_softmax_rec[2 * c + 1];
-                const float f = expf(mine.x - all.x) / all.y;
-                scale_range(out, b1, c1, f);
-            }
+            const int64_t last = todo_last[q];
+            for (int64_t p = todo_first[q]; p <= last; p += G * kSmPart * 64)
+                for (int64_t w0 = p + 64 * wave; w0 <= min(last, p + kSmPart * 64 - 1); w0 += kSmBlock)
+                    softmax_row_batch(row_ptr, x, out, w0, last, lane);
         }
     }
+    for (int64_t i = blockIdx.x; i < n_huge; i += G)
+        softmax_merge_chunk(row_ptr, out, g_softmax_rec, g_softmax_rows, g_softmax_list[n_chunks + 1 - i] & kSmListChunk);
 }
 
 // SpMM Y[r, :] = sum_p x[p] * H[col_p, :] over a CSR pattern.  Every wave owns kChunk consecutive
@@ -685,7 +698,7 @@ static int softmax_store(float2 **rec, int4 **rows, int32_t **list)
 int64_t row_softmax_workspace_bytes(int64_t nnz)
 {
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    return (((n_chunks * 36 + 4) + 255) / 256) * 256;  // two float2, one int4 and one list item per chunk, and the list's count
+    return (((n_chunks * 36 + 8) + 255) / 256) * 256;  // two float2, one int4 and one list item per chunk, and the two lists' lengths
 }
 
 int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_x, float *d_out, void *stream, void *d_ws, int64_t nnz)
@@ -694,7 +707,7 @@ int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_
     float2 *rec = nullptr;
     int4 *rows = nullptr;
     int32_t *list = nullptr;
-    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] chunk layouts, then the list: its count and [n_chunks] items
+    if (d_ws) {  // [2 * n_chunks] records, then [n_chunks] chunk layouts, then the two lists: their lengths and [n_chunks] items
         const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
         rec = static_cast<float2 *>(d_ws);
         rows = reinterpret_cast<int4 *>(rec + 2 * n_chunks);
