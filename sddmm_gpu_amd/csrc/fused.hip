@@ -49,38 +49,48 @@ static __device__ __align__(256) int4 g_softmax_rows_store[kSmMaxChunks];
 // other from [n_chunks + 1] downwards (a chunk is in one of them at most)
 static __device__ __align__(256) int32_t g_softmax_list_store[kSmMaxChunks + 64];
 
-// First kernel: the layout, one thread per chunk (two binary searches of row_ptr whose loads the other
+// First kernel: the layout, one thread per chunk (a binary search of row_ptr whose loads the other
 // threads' searches hide).  With r the row that holds entry c * kSmChunk, chunk c begins at r's first
 // entry (r short), after r's last (r long; the chunk may come out empty) or at entry c * kSmChunk itself
 // (r huge); it ends where chunk c + 1 would begin if that row were short (so a long row that starts
-// past the chunk's rows is left out) or at the multiple (huge).
+// past the chunk's rows is left out) or at the multiple (huge).  The row of chunk c + 1 is the next
+// thread's search: a workgroup of 256 threads lays out 255 chunks (the kernel is bound by the number of
+// its scattered loads).
 __global__ __launch_bounds__(256)
 void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, int4 *__restrict__ g_softmax_rows,
                                    int32_t *__restrict__ g_softmax_list)
 {
+    __shared__ int row_of[256], begin_of[256], end_of[256];  // the row that holds a chunk's first entry, and its extent
     if (blockIdx.x == 0 && threadIdx.x < 2) g_softmax_list[threadIdx.x] = 0;  // (the third kernel counts in them)
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < n_chunks; c += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t p0 = c * kSmChunk, p1 = min(nnz - 1, p0 + kSmChunk);  // (p1 = nnz - 1 in the last chunk: not used there)
-        // first row whose end lies beyond p0 / p1
-        int64_t lo0 = 0, hi0 = n_rows - 1, lo1 = 0, hi1 = n_rows - 1;
-        while (lo0 < hi0 || lo1 < hi1) {
-            if (lo0 < hi0) { const int64_t mid = (lo0 + hi0) >> 1; if (row_ptr[mid + 1] <= p0) lo0 = mid + 1; else hi0 = mid; }
-            if (lo1 < hi1) { const int64_t mid = (lo1 + hi1) >> 1; if (row_ptr[mid + 1] <= p1) lo1 = mid + 1; else hi1 = mid; }
+    for (int64_t base = (int64_t)blockIdx.x * 255; base < n_chunks; base += (int64_t)gridDim.x * 255) {
+        const int64_t c = base + threadIdx.x, p0 = c * kSmChunk;
+        int64_t lo0 = 0, b0 = 0, e0 = 0;
+        if (c < n_chunks) {
+            int64_t hi0 = n_rows - 1;  // first row whose end lies beyond p0
+            while (lo0 < hi0) {
+                const int64_t mid = (lo0 + hi0) >> 1;
+                if (row_ptr[mid + 1] <= p0) lo0 = mid + 1; else hi0 = mid;
+            }
+            b0 = row_ptr[lo0];
+            e0 = row_ptr[lo0 + 1];
         }
+        __syncthreads();  // (the round before has read its neighbours' rows)
+        row_of[threadIdx.x] = (int)lo0; begin_of[threadIdx.x] = (int)b0; end_of[threadIdx.x] = (int)e0;
+        __syncthreads();
+        if (c >= n_chunks || threadIdx.x == 255) continue;
         int4 lay;
-        const int64_t b0 = row_ptr[lo0], e0 = row_ptr[lo0 + 1];
         const int k0 = softmax_row_class(e0 - b0);
         lay.x = (int)(k0 == 0 ? b0 : k0 == 1 ? e0 : p0);
         lay.z = (int)(k0 == 1 ? lo0 + 1 : lo0);
         if (p0 + kSmChunk >= nnz) {
             lay.y = (int)nnz;
             lay.w = (int)(n_rows - 1);
-        } else {
-            const int64_t b1 = row_ptr[lo1], e1 = row_ptr[lo1 + 1];
+        } else {  // (chunk c + 1 exists: its first entry p0 + kSmChunk is an entry)
+            const int64_t lo1 = row_of[threadIdx.x + 1], b1 = begin_of[threadIdx.x + 1], e1 = end_of[threadIdx.x + 1];
             const int k1 = softmax_row_class(e1 - b1);
-            lay.y = (int)(k1 == 2 ? p1 : b1);
+            lay.y = (int)(k1 == 2 ? p0 + kSmChunk : b1);
             lay.w = (int)(k1 == 2 ? lo1 : lo1 - 1);
         }
         g_softmax_rows[c] = lay;
