@@ -24,8 +24,10 @@ namespace {
 //   huge rows (beyond that) are cut at the multiples of kSmChunk: a workgroup takes a piece, stores it
 //        as exp(x - m) with the piece's own maximum m and leaves (m, sum) in a record of the chunk; a last
 //        kernel merges the records of each huge row and scales its pieces.
-// The first kernel lays the chunks out (one thread per chunk); all kernels read the number of entries
-// from row_ptr[n_rows] on the device and walk the chunks with a grid-sized stride.  No LDS staging: a
+// Three kernels: the first lays the chunks out (one thread per chunk); the second takes the short rows
+// with two thirds of its workgroups and the long rows and pieces with the others; the last works from two
+// lists that the second makes.  All read the number of entries from row_ptr[n_rows] on the device and walk
+// the chunks with a grid-sized stride.  No LDS staging: a
 // row's loads are all in flight together, and 16 waves per compute unit hide their latency.
 constexpr int kSmChunk = 4096;
 constexpr int kSmBlock = 256;
@@ -61,7 +63,7 @@ void sddmm_row_softmax_rows_kernel(const int32_t *__restrict__ row_ptr, int64_t 
                                    int32_t *__restrict__ g_softmax_list)
 {
     __shared__ int row_of[256], begin_of[256], end_of[256];  // the row that holds a chunk's first entry, and its extent
-    if (blockIdx.x == 0 && threadIdx.x < 2) g_softmax_list[threadIdx.x] = 0;  // (the third kernel counts in them)
+    if (blockIdx.x == 0 && threadIdx.x < 2) g_softmax_list[threadIdx.x] = 0;  // (the second kernel counts in them)
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     for (int64_t base = (int64_t)blockIdx.x * 255; base < n_chunks; base += (int64_t)gridDim.x * 255) {
@@ -249,17 +251,16 @@ __device__ __forceinline__ void softmax_row_batch(const int32_t *__restrict__ ro
         }
 }
 
-// Second kernel: the short rows, a wave per chunk.
-__global__ __launch_bounds__(kSmBlock, 4)  // (at least four waves per SIMD; it takes 80 registers, so six fit)
-void sddmm_row_softmax_short_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                    const int4 *__restrict__ g_softmax_rows)
+// The short rows, a wave per chunk; workgroup `group` of `n_groups`.
+__device__ __forceinline__ void softmax_short_rows(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                                   const int4 *__restrict__ g_softmax_rows, int64_t group, int64_t n_groups)
 {
     const int lane = threadIdx.x & 63;
     const int64_t nnz = row_ptr[n_rows];
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
-    const int64_t n_waves = (int64_t)gridDim.x * (kSmBlock / 64);
+    const int64_t n_waves = n_groups * (kSmBlock / 64);
     const int64_t own = softmax_own_batches(n_rows, n_chunks);
-    for (int64_t c = (int64_t)blockIdx.x * (kSmBlock / 64) + (threadIdx.x >> 6); c < n_chunks; c += n_waves) {
+    for (int64_t c = group * (kSmBlock / 64) + (threadIdx.x >> 6); c < n_chunks; c += n_waves) {
         const int4 lay = g_softmax_rows[c];
         if (lay.x >= lay.y) continue;
         const int64_t last = min((int64_t)lay.w, (int64_t)lay.z + 64 * own - 1);
@@ -354,15 +355,15 @@ __device__ __forceinline__ void softmax_long_row(const float *x, float *out, int
     // (the next row writes its maxima after this row's second barrier and its sums after its own first: no barrier needed here)
 }
 
-// Third kernel: the long rows and the pieces of huge rows.  A long row holds the multiple of kSmChunk
+// The long rows and the pieces of huge rows; workgroup `group` of `n_groups`.  A long row holds the multiple of kSmChunk
 // that follows its first entry, so it is the row after the last row of the chunk whose window
 // [c * kSmChunk, (c + 1) * kSmChunk) it starts in; a huge row is the first or the last row of every chunk
-// it touches.  Workgroup b looks at the chunks b, b + grid, ...: first at many of them at once, a thread
+// it touches.  Workgroup b looks at the chunks b, b + n_groups, ...: first at many of them at once, a thread
 // per chunk (a few dependent loads each, which a walk chunk by chunk would pay for one after the other),
 // what it finds collected in a list; then the list item by item.
-__global__ __launch_bounds__(kSmBlock, 4)  // (four waves per SIMD: four rows in flight per compute unit)
-void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
-                                   float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows, int32_t *g_softmax_list)
+__device__ __forceinline__ void softmax_long_rows(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                                  float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows, int32_t *g_softmax_list,
+                                                  int64_t group, int64_t n_groups)
 {
     __shared__ float red[2 * kSmBlock / 64];
     __shared__ int4 todo[3 * kSmBlock];  // first entry, end, record (-1: a whole row)
@@ -371,11 +372,11 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
     const int64_t n_chunks = (nnz + kSmChunk - 1) / kSmChunk;
     const bool vec_in = (reinterpret_cast<uintptr_t>(x) & 15u) == 0, vec_out = (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     const int64_t own = softmax_own_batches(n_rows, n_chunks);
-    for (int64_t base = blockIdx.x; base < n_chunks; base += (int64_t)gridDim.x * kSmBlock) {
+    for (int64_t base = group; base < n_chunks; base += n_groups * kSmBlock) {
         __syncthreads();  // the list of the round before has been worked off
         if (threadIdx.x == 0) n_todo = 0;
         __syncthreads();
-        const int64_t c = base + (int64_t)threadIdx.x * gridDim.x;
+        const int64_t c = base + (int64_t)threadIdx.x * n_groups;
         int item = 0;  // this chunk's item of the last kernel's lists, if it has one
         if (c < n_chunks) {
             const int4 lay = g_softmax_rows[c];
@@ -434,6 +435,19 @@ void sddmm_row_softmax_long_kernel(const int32_t *__restrict__ row_ptr, int64_t 
             else softmax_long_row<kSmLongQ>(x, out, rb, re, nnz, vec_in, vec_out, red, rec);
         }
     }
+}
+
+// Second kernel: every third workgroup takes the long rows, the others the short ones; the two kinds of
+// work fill each other's gaps (a long row's workgroup loads, then reduces, then stores).
+__global__ __launch_bounds__(kSmBlock, 4)  // (four waves per SIMD: four long rows in flight per compute unit)
+void sddmm_row_softmax_main_kernel(const int32_t *__restrict__ row_ptr, int64_t n_rows, const float *x, float *out,
+                                   float2 *g_softmax_rec, const int4 *__restrict__ g_softmax_rows, int32_t *g_softmax_list)
+{
+    // (a third for the long rows: measured against a half and a quarter on a recommender and an R-MAT pattern)
+    constexpr int every = 3;
+    const int64_t n_long = (gridDim.x + every - 1) / every, mine = blockIdx.x / every;
+    if (blockIdx.x % every == 0) softmax_long_rows(row_ptr, n_rows, x, out, g_softmax_rec, g_softmax_rows, g_softmax_list, mine, n_long);
+    else softmax_short_rows(row_ptr, n_rows, x, out, g_softmax_rows, blockIdx.x - mine - 1, gridDim.x - n_long);
 }
 
 // (m, sum) of the huge row [rb, re) from the records of the chunks it spans: the last-slot record of its
@@ -497,7 +511,7 @@ __device__ __forceinline__ void softmax_merge_chunk(const int32_t *__restrict__ 
     }
 }
 
-// Last kernel, over the two lists that the third kernel made.
+// Last kernel, over the two lists that the second kernel made.
 //  - The chunks whose own wave left batches of rows.  Every workgroup reads that whole list, kSmBlock items
 //    at a time (on most matrices it is empty), and takes its share: a chunk's further batches in parts of
 //    kSmPart (one or two per wave of a workgroup), part p of list item i with the workgroup (i + p) mod
@@ -728,9 +742,7 @@ int launch_row_softmax(int64_t n_rows, const int32_t *d_row_ptr, const float *d_
     // (the entry count lives on the device: the grids are sized for the machine, the kernels stride over the chunks)
     const unsigned grid = 256 * 4;
     hipLaunchKernelGGL(sddmm_row_softmax_rows_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_row_ptr, n_rows, rows, list);
-    hipLaunchKernelGGL(sddmm_row_softmax_short_kernel, dim3(4 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
-                       (const int4 *)rows);
-    hipLaunchKernelGGL(sddmm_row_softmax_long_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
+    hipLaunchKernelGGL(sddmm_row_softmax_main_kernel, dim3(6 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x, d_out,
                        rec, (const int4 *)rows, list);
     hipLaunchKernelGGL(sddmm_row_softmax_merge_kernel, dim3(2 * grid), dim3(kSmBlock), 0, (hipStream_t)stream, d_row_ptr, n_rows, d_x,
                        d_out, (const float2 *)rec, (const int4 *)rows, (const int32_t *)list);

@@ -150,12 +150,11 @@ void sddmm_spmm_tile_kernel(const SpmmArgs a)
 // Y[row, slice] = sum of the row's partial rows: one wave per listed row, group g takes the partial
 // rows g, g + 8, ... and the groups' sums are added across the wave.
 template <int KPL>
-__global__ __launch_bounds__(256)
-void sddmm_spmm_sum_kernel(const SpmmArgs a)
+__device__ __forceinline__ void spmm_sum_rows(const SpmmArgs &a, int64_t block)
 {
     constexpr int G = 8, K4 = G * KPL;
     const int lane = threadIdx.x & 63, l = lane & 7, g = lane >> 3;
-    const int64_t w = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int64_t w = (block * 256 + threadIdx.x) >> 6;
     if (w >= a.n_sum_rows) return;
     const int b = a.row_part_ptr[w], e = a.row_part_ptr[w + 1];
     const float4 *__restrict__ part4 = reinterpret_cast<const float4 *>(a.part);
@@ -189,12 +188,11 @@ void sddmm_spmm_sum_kernel(const SpmmArgs a)
 // lanes per row, H rows gathered from global memory, four nonzeros in flight per step; the planner lists
 // the rows longest first, so that the eight rows of a wave are about equally long.
 template <int KPL>
-__global__ __launch_bounds__(256)
-void sddmm_spmm_rows_kernel(const SpmmArgs a)
+__device__ __forceinline__ void spmm_gather_rows(const SpmmArgs &a, int64_t block)
 {
     constexpr int G = 8;
     const int lane = threadIdx.x & 63, l = lane & 7;
-    const int64_t grp = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int64_t grp = (block * 256 + threadIdx.x) >> 3;
     if (grp >= a.n_gather_rows) return;
     const int row = a.gather_rows[grp];
     const int b = a.row_ptr[row], e = a.row_ptr[row + 1];
@@ -235,6 +233,19 @@ void sddmm_spmm_rows_kernel(const SpmmArgs a)
     for (int j = 0; j < KPL; ++j) y[j * G] = acc[j];
 }
 
+// Second kernel of a slice: the sums of the partial rows (a stream through memory) and the rows outside
+// the tiles (gathers from L2) side by side, sum_blocks and gather_blocks workgroups of each spread evenly
+// over the grid, so that the two kinds of traffic overlap.
+template <int KPL>
+__global__ __launch_bounds__(256)
+void sddmm_spmm_rows_kernel(const SpmmArgs a, int64_t sum_blocks, int64_t gather_blocks)
+{
+    const int64_t i = blockIdx.x, n = sum_blocks + gather_blocks;
+    const int64_t sums_before = i * sum_blocks / n;  // (of the workgroups 0 .. i - 1)
+    if ((i + 1) * sum_blocks / n > sums_before) spmm_sum_rows<KPL>(a, sums_before);
+    else spmm_gather_rows<KPL>(a, i - sums_before);
+}
+
 }  // namespace
 
 namespace sddmm {
@@ -268,8 +279,8 @@ void launch_spmm_slice(const SpmmArgs &a, int k_slice, int nwaves, int grid, int
             if (nwaves == 12) hipLaunchKernelGGL((sddmm_spmm_tile_kernel<kpl, 12>), dim3((unsigned)grid), dim3(12 * 64), (size_t)lds_bytes, st, a); \
             else hipLaunchKernelGGL((sddmm_spmm_tile_kernel<kpl, 16>), dim3((unsigned)grid), dim3(16 * 64), (size_t)lds_bytes, st, a);              \
         }                                                                                                              \
-        if (a.n_sum_rows > 0) hipLaunchKernelGGL((sddmm_spmm_sum_kernel<kpl>), dim3(sum_grid), dim3(256), 0, st, a);         \
-        if (a.n_gather_rows > 0) hipLaunchKernelGGL((sddmm_spmm_rows_kernel<kpl>), dim3(rows_grid), dim3(256), 0, st, a);    \
+        if (sum_grid + rows_grid > 0)                                                                                  \
+            hipLaunchKernelGGL((sddmm_spmm_rows_kernel<kpl>), dim3(sum_grid + rows_grid), dim3(256), 0, st, a, (int64_t)sum_grid, (int64_t)rows_grid); \
     } while (0)
     if (k_slice == 128) SDDMM_SPMM_LAUNCH(4);
     else if (k_slice == 64) SDDMM_SPMM_LAUNCH(2);
