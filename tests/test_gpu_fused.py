@@ -43,7 +43,7 @@ def test_row_softmax_matches_oracle(oracle, cfg, scale):
 def test_row_softmax_edge_rows(oracle, misalign):
     """Rows at the boundaries of the kernel's cases: rows of up to 4096 entries are grouped into chunks of whole rows, a wave
     takes a chunk 64 rows at a time and gives a row to a lane (up to 8 entries), 8 lanes (up to 96), 32 lanes (up to 512)
-    or all its lanes (up to 1024 in registers, beyond that in two walks); longer rows have a kernel of their own (next
+    or all its lanes (up to 1024 in registers, beyond that in two walks); longer rows go to workgroups of their own (next
     test).  The runs of empty rows span several chunks' worth of row pointers."""
     lens = ([0, 1, 0, 8, 9, 64, 65, 96, 97, 192, 193, 512, 513, 1023, 1024, 1025, 0, 2, 511]      # every class, whole rows
             + [2 * 4096 - sum([1, 8, 9, 64, 65, 96, 97, 192, 193, 512, 513, 1023, 1024, 1025, 2, 511])]  # ... up to the end of chunk 1 exactly
@@ -131,6 +131,33 @@ def test_row_softmax_mostly_empty_rows(oracle):
         capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), out.data_ptr())
         torch.cuda.synchronize()
         softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
+
+
+@pytest.mark.parametrize("kind", ["heavy tail", "huge rows among empty ones", "chunks with both", "class limits"])
+def test_row_softmax_mixed_lengths(oracle, kind):
+    """Row-length mixes that put several of the pass's cases into the same chunks: a heavy-tailed distribution; rows of
+    tens of thousands of entries between long runs of empty rows; stretches of mostly empty rows that a huge row runs
+    into (the chunk is then in the last kernel's list for both reasons); rows at the limits of every class."""
+    rng = np.random.default_rng(11)
+    if kind == "heavy tail":
+        lens = np.minimum((rng.pareto(0.8, 40_000) * 3).astype(np.int64), 300_000)
+    elif kind == "huge rows among empty ones":
+        lens = np.zeros(600_000, dtype=np.int64)
+        at = rng.choice(len(lens), 200, replace=False)
+        lens[at] = rng.choice([1, 5, 100, 3000, 5000, 17_000, 40_000], 200)
+    elif kind == "chunks with both":
+        lens = np.zeros(1_500_000, dtype=np.int64)
+        lens[::len(lens) // 37] = 50_000
+        lens[5::997] = 3
+    else:
+        lens = rng.choice([4095, 4096, 4097, 8191, 8192, 8193, 16_376, 16_377, 12_288, 1, 0], 300)
+    rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    x = rng.normal(0, 6, rp[-1]).astype(np.float32)
+    dev = torch.device(DEV)
+    xd = torch.from_numpy(x).to(dev); out = torch.full_like(xd, float("nan")); rpd = torch.from_numpy(rp).to(dev)
+    capi.row_softmax(len(lens), rpd.data_ptr(), xd.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    softmax_ok(out.cpu().numpy(), oracle.row_softmax(rp, x))
 
 
 @pytest.mark.parametrize("kernel,K", [("auto", 128), ("auto", 64), ("row", 100), ("lds", 32), ("panel", 64)])
